@@ -67,8 +67,10 @@ def architecture_name(raw: Dict[str, Any]) -> str:
     """The name the registry is keyed on: config.json's architectures[0]
     (the reference detects the family from the same key, cpmcu/common/utils.py:41-42)."""
     arch = raw.get("architectures")
+    if arch is None and isinstance(raw.get("architecture"), str) and raw["architecture"]:
+        return raw["architecture"]          # some configurations name their one architecture directly
     if not isinstance(arch, list) or not arch or not isinstance(arch[0], str):
-        raise ConfigError("config.json: 'architectures' must be a non-empty list of names")
+        raise ConfigError("config.json: 'architectures' must be a non-empty list of names (or 'architecture' a name)")
     return arch[0]
 
 

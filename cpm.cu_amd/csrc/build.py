@@ -30,6 +30,9 @@ MODULES: Dict[str, List[str]] = {
     "attention": ["attention.hip"],
     "sparse": ["sparse.hip"],
     "qkv": ["qkv_rope.hip", "strip.hip"],
+    "norms": ["norms.hip"],
+    "ssm": ["ssm.hip"],
+    "attention_general": ["attention_general.hip"],
 }
 HEADERS = ["common.h"]
 # headers of single libraries

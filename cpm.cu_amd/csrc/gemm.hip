@@ -77,6 +77,83 @@ extern "C" const char* cpmcu_gemm_nt_plain(const void* X, long ldx, const void* 
     return nullptr;
 }
 
+// ---------------------------------------------------------------------------
+// The same product head by head: Y[m, h, :] = X[m, h, :] . W[h]^T for H heads with a weight [N, K] each (W is
+// [H, N, K]); head h's run of a row starts at h * hsx (X) and h * hsy (Y), so inputs and outputs may be slices
+// of wider rows.  With `gate` the rows of head h are multiplied by sigmoid(gate[m * ldg + h]) (an output gate
+// of one number a head).  blockIdx.z is the head.
+// ---------------------------------------------------------------------------
+template <typename XT, typename WT, typename OT>
+__global__ __launch_bounds__(256) void gemm_heads_kernel(const XT* __restrict__ X, long ldx, long hsx,
+                                                         const WT* __restrict__ W, OT* __restrict__ Y, long ldy,
+                                                         long hsy, const XT* __restrict__ gate, long ldg, int M, int N,
+                                                         int K) {
+    __shared__ float xs[GT_BK][GT_BM + 1];
+    __shared__ float ws[GT_BK][GT_BN + 1];
+    const int tx = threadIdx.x % 16, ty = threadIdx.x / 16;
+    const int m0 = blockIdx.y * GT_BM, n0 = blockIdx.x * GT_BN, h = blockIdx.z;
+    X += (long)h * hsx;
+    Y += (long)h * hsy;
+    W += (long)h * N * K;
+    float acc[4][4] = {};
+    for (int k0 = 0; k0 < K; k0 += GT_BK) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const int e = threadIdx.x + i * 256;
+            const int r = e / GT_BK, kk = e % GT_BK;
+            const int k = k0 + kk;
+            xs[kk][r] = (m0 + r < M && k < K) ? to_f32(X[(long)(m0 + r) * ldx + k]) : 0.f;
+            ws[kk][r] = (n0 + r < N && k < K) ? to_f32(W[(long)(n0 + r) * K + k]) : 0.f;
+        }
+        __syncthreads();
+#pragma unroll
+        for (int kk = 0; kk < GT_BK; ++kk) {
+            float a[4], b[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) a[i] = xs[kk][ty * 4 + i];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) b[j] = ws[kk][tx * 4 + j];
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int j = 0; j < 4; ++j) acc[i][j] += a[i] * b[j];
+        }
+        __syncthreads();
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int m = m0 + ty * 4 + i;
+        if (m >= M) continue;
+        float gs = 1.f;
+        if (gate) gs = 1.0f / (1.0f + expf(-to_f32(gate[(long)m * ldg + h])));
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int n = n0 + tx * 4 + j;
+            if (n < N) Y[(long)m * ldy + n] = from_f32<OT>(gs * acc[i][j]);
+        }
+    }
+}
+
+extern "C" const char* cpmcu_gemm_nt_heads(const void* X, long ldx, long hsx, const void* W, void* Y, long ldy, long hsy,
+                                           const void* gate, long ldg, int in_dtype, int out_dtype, int M, int H, int N,
+                                           int K, hipStream_t stream) {
+    CPMCU_REQUIRE(M > 0 && H > 0 && N > 0 && K > 0, "gemm_heads: empty shape M=%d heads=%d N=%d K=%d", M, H, N, K);
+    CPMCU_REQUIRE(ldx >= (H - 1) * hsx + K && ldy >= (H - 1) * hsy + N && (!gate || ldg >= H),
+                  "gemm_heads: rows of %ld / %ld elements cannot hold %d heads", ldx, ldy, H);
+    dim3 grid((N + GT_BN - 1) / GT_BN, (M + GT_BM - 1) / GT_BM, H);
+    CPMCU_REQUIRE(grid.y <= 65535 && H <= 65535, "gemm_heads: M=%d or heads=%d too large for one launch", M, H);
+#define LAUNCH(T, OT)                                                                                          \
+    gemm_heads_kernel<T, T, OT><<<grid, 256, 0, stream>>>((const T*)X, ldx, hsx, (const T*)W, (OT*)Y, ldy, hsy, \
+                                                          (const T*)gate, ldg, M, N, K)
+    if (in_dtype == CPMCU_F32 && out_dtype == CPMCU_F32) LAUNCH(float, float);
+    else if (in_dtype == CPMCU_BF16 && out_dtype == CPMCU_BF16) LAUNCH(bf16_t, bf16_t);
+    else if (in_dtype == CPMCU_BF16 && out_dtype == CPMCU_F32) LAUNCH(bf16_t, float);
+    else CPMCU_FAIL("gemm_heads: unsupported dtypes in=%d out=%d", in_dtype, out_dtype);
+#undef LAUNCH
+    CPMCU_LAUNCH_CHECK("gemm_nt_heads");
+    return nullptr;
+}
+
 // ===========================================================================
 // Skinny product for decode steps (bf16, at most 64 rows of X):
 //   Y[m,N] = alpha * X[m,K] . W[N,K]^T

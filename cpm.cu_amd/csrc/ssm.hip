@@ -1,0 +1,202 @@
+// State-space (Mamba-2 style) sequence mixing over a packed batch, with per-slot state:
+//
+//  * conv_silu_kernel: causal convolution per channel over a sequence's tokens (taps weights a channel, the last
+//    column is the current token's; inputs before the sequence's start are zero) followed by SiLU.  The
+//    sequence's last taps-1 inputs live in the slot's state, so a step continues where the last one ended.
+//  * conv_state_kernel: moves the step's last inputs into that state (after the convolution has read it).
+//  * ssm_scan_kernel: the recurrence, per head h (group g = h / (heads / groups)):
+//        dt_t = softplus(raw_t + dt_bias_h)             (no clamp)
+//        S_t  = exp(-exp(A_log_h) * dt_t) * S_(t-1) + dt_t * B_t x_t^T        S: [state N, head size P]
+//        y_t  = S_t^T C_t + D_h x_t
+//    all in float, the state in float in the slot, carried from step to step.
+//
+// The scan walks a sequence's tokens in order; a workgroup owns one (sequence, head, 32 columns of P), a
+// column's N state values are spread over 8 neighbouring lanes, and the tokens' B, C, x and dt pass through
+// LDS in tiles of 16 tokens.
+#include "common.h"
+
+__device__ inline float silu_f(float z) { return z / (1.0f + expf(-z)); }
+
+// grid (sequences, token tiles of 64, channel blocks of 256 threads)
+template <typename UT>
+__global__ __launch_bounds__(256) void conv_silu_kernel(const UT* __restrict__ u, long ldu,
+                                                        const float* __restrict__ weight,
+                                                        const float* __restrict__ bias,
+                                                        const float* __restrict__ state, float* __restrict__ out,
+                                                        const int* __restrict__ cu_q, const int* __restrict__ seq_slot,
+                                                        int C, int taps) {
+    const int b = blockIdx.x;
+    const int start = cu_q[b], q = cu_q[b + 1] - start;
+    const int slot = seq_slot[b];
+    const int c = blockIdx.z * blockDim.x + threadIdx.x;
+    if (c >= C) return;
+    const int i0 = blockIdx.y * 64, i1 = min(i0 + 64, q);
+    const float* st = state + (long)slot * (taps - 1) * C + c;        // [slot][taps-1][C]
+    const float bs = bias ? bias[c] : 0.f;
+    for (int i = i0; i < i1; ++i) {
+        float acc = bs;
+        for (int k = 0; k < taps; ++k) {
+            const int j = i - (taps - 1 - k);                          // local index of the input this tap reads
+            const float in = j >= 0 ? to_f32(u[(long)(start + j) * ldu + c]) : st[(long)(taps - 1 + j) * C];
+            acc += weight[(long)c * taps + k] * in;
+        }
+        out[(long)(start + i) * C + c] = silu_f(acc);
+    }
+}
+
+// grid (sequences, channel blocks): state[j] <- the input at local index q - (taps-1) + j, which is one of the
+// step's tokens or, for a short step, an older entry of the state (read before it is overwritten: a thread
+// walks j upwards and reads index j + q > j).
+template <typename UT>
+__global__ __launch_bounds__(256) void conv_state_kernel(const UT* __restrict__ u, long ldu, float* __restrict__ state,
+                                                         const int* __restrict__ cu_q, const int* __restrict__ seq_slot,
+                                                         int C, int taps) {
+    const int b = blockIdx.x;
+    const int start = cu_q[b], q = cu_q[b + 1] - start;
+    const int slot = seq_slot[b];
+    const int c = blockIdx.y * blockDim.x + threadIdx.x;
+    if (c >= C) return;
+    float* st = state + (long)slot * (taps - 1) * C + c;
+    for (int j = 0; j < taps - 1; ++j) {
+        const int i = q - (taps - 1) + j;
+        st[(long)j * C] = i >= 0 ? to_f32(u[(long)(start + i) * ldu + c]) : st[(long)(j + q) * C];
+    }
+}
+
+extern "C" const char* cpmcu_conv_silu(const void* u, long ldu, int u_dtype, const float* weight, const float* bias,
+                                       float* state, float* out, const int* cu_q, const int* seq_slot, int n_seqs,
+                                       int max_q, int C, int taps, int update_state, hipStream_t stream) {
+    CPMCU_REQUIRE(n_seqs > 0 && max_q > 0 && C > 0 && taps >= 1, "conv_silu: empty shape sequences=%d tokens=%d channels=%d taps=%d",
+                  n_seqs, max_q, C, taps);
+    CPMCU_REQUIRE(ldu >= C, "conv_silu: rows of %ld elements cannot hold %d channels", ldu, C);
+    CPMCU_REQUIRE(taps == 1 || state, "conv_silu: the state of the last inputs is missing");
+    const int cb = (C + 255) / 256, tb = (max_q + 63) / 64;
+    CPMCU_REQUIRE(tb <= 65535 && cb <= 65535, "conv_silu: shape exceeds the launch grid");
+    dim3 grid(n_seqs, tb, cb), grid2(n_seqs, cb);
+    if (u_dtype == CPMCU_F32) {
+        conv_silu_kernel<float><<<grid, 256, 0, stream>>>((const float*)u, ldu, weight, bias, state, out, cu_q, seq_slot, C, taps);
+        if (update_state && taps > 1)
+            conv_state_kernel<float><<<grid2, 256, 0, stream>>>((const float*)u, ldu, state, cu_q, seq_slot, C, taps);
+    } else if (u_dtype == CPMCU_BF16) {
+        conv_silu_kernel<bf16_t><<<grid, 256, 0, stream>>>((const bf16_t*)u, ldu, weight, bias, state, out, cu_q, seq_slot, C, taps);
+        if (update_state && taps > 1)
+            conv_state_kernel<bf16_t><<<grid2, 256, 0, stream>>>((const bf16_t*)u, ldu, state, cu_q, seq_slot, C, taps);
+    } else {
+        CPMCU_FAIL("conv_silu: unknown dtype %d", u_dtype);
+    }
+    CPMCU_LAUNCH_CHECK("conv_silu");
+    return nullptr;
+}
+
+#define SCAN_PB 32       // columns of P a workgroup
+#define SCAN_L 8         // lanes a column: state index n = l + 8 i
+#define SCAN_TT 16       // tokens a tile in LDS
+
+__device__ inline float softplus_f(float v) { return fmaxf(v, 0.f) + log1pf(expf(-fabsf(v))); }
+
+// xbc: float [n, ldx] = [x: heads*P | B: groups*N | C: groups*N]; dt: raw step sizes [n, lddt] (first `heads`
+// columns at the given pointer); state: float [slots][heads][P][N]; y: float [n, heads*P].
+template <int NR, typename DT>
+__global__ __launch_bounds__(256) void ssm_scan_kernel(const float* __restrict__ xbc, long ldx,
+                                                       const DT* __restrict__ dt, long lddt,
+                                                       const float* __restrict__ dt_bias,
+                                                       const float* __restrict__ A_log, const float* __restrict__ Dskip,
+                                                       float* __restrict__ state, float* __restrict__ y,
+                                                       const int* __restrict__ cu_q, const int* __restrict__ seq_slot,
+                                                       int heads, int P, int N, int groups, int write_state) {
+    __shared__ float Bs[SCAN_TT][NR * SCAN_L];
+    __shared__ float Cs[SCAN_TT][NR * SCAN_L];
+    __shared__ float xs[SCAN_TT][SCAN_PB];
+    __shared__ float dts[SCAN_TT], das[SCAN_TT];
+    const int b = blockIdx.x, h = blockIdx.y, p0 = blockIdx.z * SCAN_PB;
+    const int start = cu_q[b], q = cu_q[b + 1] - start;
+    const int slot = seq_slot[b];
+    const int g = h / (heads / groups);
+    const int inner = heads * P;
+    const int pl = threadIdx.x / SCAN_L, l = threadIdx.x % SCAN_L;
+    const int p = p0 + pl;
+    const bool p_ok = p < P;
+    float S[NR];
+    float* sp = state + (((long)slot * heads + h) * P + (p_ok ? p : 0)) * N;
+#pragma unroll
+    for (int i = 0; i < NR; ++i) {
+        const int n = l + SCAN_L * i;
+        S[i] = (p_ok && n < N) ? sp[n] : 0.f;
+    }
+    const float A = expf(A_log[h]), bias = dt_bias[h], Dh = Dskip[h];
+    for (int t0 = 0; t0 < q; t0 += SCAN_TT) {
+        const int tn = min(SCAN_TT, q - t0);
+        __syncthreads();
+        for (int e = threadIdx.x; e < tn * NR * SCAN_L; e += 256) {
+            const int tt = e / (NR * SCAN_L), n = e % (NR * SCAN_L);
+            const float* row = xbc + (long)(start + t0 + tt) * ldx + inner + (long)g * N;
+            Bs[tt][n] = n < N ? row[n] : 0.f;
+            Cs[tt][n] = n < N ? row[(long)groups * N + n] : 0.f;
+        }
+        for (int e = threadIdx.x; e < tn * SCAN_PB; e += 256) {
+            const int tt = e / SCAN_PB, pp = e % SCAN_PB;
+            xs[tt][pp] = p0 + pp < P ? xbc[(long)(start + t0 + tt) * ldx + (long)h * P + p0 + pp] : 0.f;
+        }
+        if ((int)threadIdx.x < tn) {
+            const float d = softplus_f(to_f32(dt[(long)(start + t0 + threadIdx.x) * lddt + h]) + bias);
+            dts[threadIdx.x] = d;
+            das[threadIdx.x] = expf(-A * d);
+        }
+        __syncthreads();
+        for (int tt = 0; tt < tn; ++tt) {
+            const float d = dts[tt], da = das[tt], xv = xs[tt][pl];
+            const float dx = d * xv;
+            float acc = 0.f;
+#pragma unroll
+            for (int i = 0; i < NR; ++i) {
+                const int n = l + SCAN_L * i;
+                S[i] = da * S[i] + dx * Bs[tt][n];
+                acc += S[i] * Cs[tt][n];
+            }
+            // the column's 8 lanes are neighbours: sum inside the vector unit
+            acc += CPMCU_DPP(acc, 0xB1);
+            acc += CPMCU_DPP(acc, 0x4E);
+            acc += CPMCU_DPP(acc, 0x141);
+            if (l == 0 && p_ok) y[(long)(start + t0 + tt) * inner + (long)h * P + p] = acc + Dh * xv;
+        }
+    }
+    if (write_state && p_ok) {
+#pragma unroll
+        for (int i = 0; i < NR; ++i) {
+            const int n = l + SCAN_L * i;
+            if (n < N) sp[n] = S[i];
+        }
+    }
+}
+
+extern "C" const char* cpmcu_ssm_scan(const float* xbc, long ldx, const void* dt, long lddt, int dt_dtype,
+                                      const float* dt_bias, const float* A_log, const float* Dskip, float* state,
+                                      float* y, const int* cu_q, const int* seq_slot, int n_seqs, int heads, int P,
+                                      int N, int groups, int write_state, hipStream_t stream) {
+    CPMCU_REQUIRE(n_seqs > 0 && heads > 0 && P > 0 && N > 0 && groups > 0, "ssm_scan: empty shape");
+    CPMCU_REQUIRE(heads % groups == 0, "ssm_scan: %d heads are not a multiple of %d groups", heads, groups);
+    CPMCU_REQUIRE(N <= 256, "ssm_scan: a state of %d values a column is not supported (at most 256)", N);
+    CPMCU_REQUIRE(ldx >= (long)heads * P + 2L * groups * N && lddt >= heads, "ssm_scan: rows too short");
+    const int pb = (P + SCAN_PB - 1) / SCAN_PB;
+    CPMCU_REQUIRE(heads <= 65535 && pb <= 65535, "ssm_scan: shape exceeds the launch grid");
+    dim3 grid(n_seqs, heads, pb);
+    const int need = (N + SCAN_L - 1) / SCAN_L;
+#define LAUNCH(NRv, DTv)                                                                                          \
+    ssm_scan_kernel<NRv, DTv><<<grid, 256, 0, stream>>>(xbc, ldx, (const DTv*)dt, lddt, dt_bias, A_log, Dskip, state, \
+                                                        y, cu_q, seq_slot, heads, P, N, groups, write_state)
+#define BY_NR(DTv)                          \
+    do {                                    \
+        if (need <= 2) LAUNCH(2, DTv);      \
+        else if (need <= 4) LAUNCH(4, DTv); \
+        else if (need <= 8) LAUNCH(8, DTv); \
+        else if (need <= 16) LAUNCH(16, DTv); \
+        else LAUNCH(32, DTv);               \
+    } while (0)
+    if (dt_dtype == CPMCU_F32) BY_NR(float);
+    else if (dt_dtype == CPMCU_BF16) BY_NR(bf16_t);
+    else CPMCU_FAIL("ssm_scan: unknown dtype %d", dt_dtype);
+#undef BY_NR
+#undef LAUNCH
+    CPMCU_LAUNCH_CHECK("ssm_scan");
+    return nullptr;
+}

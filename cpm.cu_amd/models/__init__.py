@@ -1,3 +1,4 @@
 """Model files.  Importing this package registers the built-in architectures."""
 from .decoder import DecoderModel, Run, sequential_schedule
 from . import minicpm
+from . import duvulix

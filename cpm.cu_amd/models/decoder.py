@@ -18,7 +18,7 @@ from typing import List, Optional, Sequence
 import torch
 
 from ..cache.paged import CacheNeeds
-from ..parts.base import Block, Norm, Part, ResidualStream, Runtime, StepContext
+from ..parts.base import Block, Norm, Part, ResidualStream, Runtime, StepContext, branch_for
 from ..parts.embedding import LMHead, TokenEmbedding
 
 
@@ -84,6 +84,6 @@ class DecoderModel(Part):
         if ctx.logit_rows is None or ctx.logit_rows.numel() == 0:
             return None
         with ctx.timed("head"):
-            y = self.final_norm.forward(stream.x, stream.pending, stream.pending_scale, ctx, rows=ctx.logit_rows,
-                                        tag="final.y")
+            y = self.final_norm.forward(stream.x, branch_for(self.final_norm, stream.take_pending()),
+                                        stream.pending_scale, ctx, rows=ctx.logit_rows, tag="final.y")
             return self.head.forward(y, ctx)

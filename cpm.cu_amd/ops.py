@@ -447,6 +447,219 @@ def sparse_select(q: torch.Tensor, ckpool: torch.Tensor, nh: int, nkv: int, hd: 
         c_long(scratch.numel() if scratch is not None else 0), _stream()))
 
 
+def _ld(t: torch.Tensor, name: str) -> int:
+    """Row stride of a 2-D tensor whose rows are contiguous (a slice of columns of a wider tensor is)."""
+    if not isinstance(t, torch.Tensor) or t.device.type != "cuda":
+        raise KernelError(f"{name}: a GPU tensor is needed (no CPU path exists)")
+    if t.dim() != 2 or (t.shape[1] > 1 and t.stride(1) != 1):
+        raise KernelError(f"{name}: rows must be contiguous, strides {tuple(t.stride())} for shape {tuple(t.shape)}")
+    return int(t.stride(0)) if t.shape[0] > 1 else max(int(t.stride(0)), int(t.shape[1]))
+
+
+def rms_norm_groups(x: torch.Tensor, weight: Optional[torch.Tensor], eps: float, out: torch.Tensor, groups: int = 1,
+                    gate: Optional[torch.Tensor] = None):
+    """out[r] = v / sqrt(mean(v^2) + eps) * weight, group by group (``groups`` equal parts of a row, each by its
+    own root mean square), v = x * silu(gate) when a gate is given (the gate comes before the norm).  x, gate
+    and out may be column slices of wider tensors; statistics in float."""
+    ldx, ldo = _ld(x, "norm x"), _ld(out, "norm out")
+    n, width = x.shape
+    if groups <= 0 or width % groups:
+        raise KernelError(f"rms_norm_groups: {width} columns do not split into {groups} equal groups")
+    if tuple(out.shape) != (n, width):
+        raise KernelError(f"norm out: shape {tuple(out.shape)}, expected {(n, width)}")
+    if weight is not None:
+        _need(weight, "norm weight", torch.float32, (width,))
+    ldz = 0
+    if gate is not None:
+        ldz = _ld(gate, "norm gate")
+        if tuple(gate.shape) != (n, width):
+            raise KernelError(f"norm gate: shape {tuple(gate.shape)}, expected {(n, width)}")
+    _check(_fn("norms", "cpmcu_rms_norm_groups")(_p(x), c_long(ldx), c_int(_code(x)), _p(gate), c_long(ldz),
+                                                 c_int(_code(gate) if gate is not None else 0), _p(weight), _p(out),
+                                                 c_long(ldo), c_int(_code(out)), c_int(n), c_int(groups),
+                                                 c_int(width // groups), c_float(eps), _stream()))
+
+
+def branch_norm_add_norm(x: torch.Tensor, branch: torch.Tensor, branch_weight: torch.Tensor, branch_eps: float,
+                         weight: Optional[torch.Tensor], eps: float, out: Optional[torch.Tensor],
+                         rows: Optional[torch.Tensor] = None):
+    """x += rmsnorm(branch) * branch_weight (in place; the branch summed over its leading axis first if it is
+    [P,n,H]); out = rmsnorm(x) * weight.  With ``rows`` (int32 [R]) only those rows are computed, into out
+    [R,H], and x is left as it was.  out None: only the residual is updated."""
+    _need(x, "norm x", torch.float32, (None, None))
+    n, H = x.shape
+    nparts, stride = 1, 0
+    if branch.dim() == 3:
+        _need(branch, "norm branch", shape=(None, n, H))
+        nparts, stride = branch.shape[0], n * H
+    else:
+        _need(branch, "norm branch", shape=(n, H))
+    _need(branch_weight, "branch norm weight", torch.float32, (H,))
+    n_out = n
+    if rows is not None:
+        _need(rows, "norm rows", torch.int32, (None,))
+        n_out = rows.shape[0]
+    if out is not None:
+        _need(weight, "norm weight", torch.float32, (H,))
+        _need(out, "norm out", shape=(n_out, H))
+    _check(_fn("norms", "cpmcu_branch_norm_add_norm")(_p(x), _p(branch), c_int(_code(branch)), c_int(nparts),
+                                                      c_long(stride), _p(branch_weight), c_float(branch_eps),
+                                                      _p(weight), c_float(eps), _p(out),
+                                                      c_int(_code(out) if out is not None else 0), _p(rows),
+                                                      c_int(n_out), c_int(H), _stream()))
+
+
+def poly_norm(z: torch.Tensor, coef: torch.Tensor, eps: float, out: torch.Tensor):
+    """out = a z/rms(z) + b z^2/rms(z^2) + c z^3/rms(z^3) + e row by row, (a, b, c, e) = coef (float32 [4] on the
+    device), powers element by element, rms(v) = sqrt(mean(v^2) + eps); z [n,F] or float partial sums [P,n,F]."""
+    nparts, stride = 1, 0
+    if z.dim() == 3:
+        _need(z, "poly_norm z", torch.float32, (None, None, None))
+        nparts, n, F = z.shape
+        stride = n * F
+    else:
+        _need(z, "poly_norm z", shape=(None, None))
+        n, F = z.shape
+    _need(coef, "poly_norm coefficients", torch.float32, (4,))
+    _need(out, "poly_norm out", shape=(n, F))
+    _check(_fn("norms", "cpmcu_poly_norm")(_p(z), c_int(_code(z)), c_int(nparts), c_long(stride), _p(coef), _p(out),
+                                           c_int(_code(out)), c_int(n), c_int(F), c_float(eps), _stream()))
+
+
+def conv_silu(u: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor], state: Optional[torch.Tensor],
+              out: torch.Tensor, cu_q: torch.Tensor, seq_slot: torch.Tensor, max_q: int, update_state: bool = True):
+    """Causal convolution per channel over each sequence's tokens, then SiLU.  u [n,C] (may be a column slice),
+    weight float32 [C,taps] (last column = the current token's), state float32 [slots, taps-1, C] = each slot's
+    last inputs (zeros before a sequence's start), out float32 [n,C].  cu_q int32 [B+1], seq_slot int32 [B];
+    max_q: the longest run of tokens a sequence brings.  The state moves on to the step's last inputs."""
+    ldu = _ld(u, "conv input")
+    n, C = u.shape
+    _need(weight, "conv weight", torch.float32, (C, None))
+    taps = weight.shape[1]
+    if bias is not None:
+        _need(bias, "conv bias", torch.float32, (C,))
+    if taps > 1:
+        _need(state, "conv state", torch.float32, (None, taps - 1, C))
+    _need(out, "conv out", torch.float32, (n, C))
+    _need(cu_q, "conv sequence starts", torch.int32, (None,))
+    B = cu_q.shape[0] - 1
+    _need(seq_slot, "conv sequence slots", torch.int32, (B,))
+    _check(_fn("ssm", "cpmcu_conv_silu")(_p(u), c_long(ldu), c_int(_code(u)), _p(weight), _p(bias), _p(state), _p(out),
+                                         _p(cu_q), _p(seq_slot), c_int(B), c_int(max_q), c_int(C), c_int(taps),
+                                         c_int(1 if update_state else 0), _stream()))
+
+
+def ssm_scan(xbc: torch.Tensor, dt: torch.Tensor, dt_bias: torch.Tensor, A_log: torch.Tensor, D: torch.Tensor,
+             state: torch.Tensor, y: torch.Tensor, cu_q: torch.Tensor, seq_slot: torch.Tensor, heads: int, P: int,
+             N: int, groups: int, write_state: bool = True):
+    """The state-space recurrence over each sequence's tokens, in float: per head h (group h // (heads/groups)),
+    d = softplus(dt + dt_bias[h]); S <- exp(-exp(A_log[h]) d) S + d B x^T; y = S^T C + D[h] x.
+    xbc float32 [n, heads*P + 2*groups*N] = [x | B | C]; dt [n, heads] (may be a column slice);
+    state float32 [slots, heads, P, N]; y float32 [n, heads*P]."""
+    _need(xbc, "scan inputs", torch.float32, (None, heads * P + 2 * groups * N))
+    n = xbc.shape[0]
+    lddt = _ld(dt, "scan step sizes")
+    if tuple(dt.shape) != (n, heads):
+        raise KernelError(f"scan step sizes: shape {tuple(dt.shape)}, expected {(n, heads)}")
+    for t, name in ((dt_bias, "dt_bias"), (A_log, "A_log"), (D, "D")):
+        _need(t, f"scan {name}", torch.float32, (heads,))
+    _need(state, "scan state", torch.float32, (None, heads, P, N))
+    _need(y, "scan out", torch.float32, (n, heads * P))
+    _need(cu_q, "scan sequence starts", torch.int32, (None,))
+    B = cu_q.shape[0] - 1
+    _need(seq_slot, "scan sequence slots", torch.int32, (B,))
+    _check(_fn("ssm", "cpmcu_ssm_scan")(_p(xbc), c_long(xbc.shape[1]), _p(dt), c_long(lddt), c_int(_code(dt)),
+                                        _p(dt_bias), _p(A_log), _p(D), _p(state), _p(y), _p(cu_q), _p(seq_slot),
+                                        c_int(B), c_int(heads), c_int(P), c_int(N), c_int(groups),
+                                        c_int(1 if write_state else 0), _stream()))
+
+
+ROTATE_TO_ROWS, ROTATE_TO_KEYS, ROTATE_TO_VALUES = 0, 1, 2
+
+
+def rotate_copy(src: torch.Tensor, src_off: int, src_head_stride: int, heads: int, width: int, rot_dims: int,
+                positions: torch.Tensor, inv_freq: Optional[torch.Tensor], mag: float, dst: torch.Tensor,
+                mode: int = ROTATE_TO_ROWS, dst_off: int = 0, dst_head_stride: int = 0,
+                tok_slot: Optional[torch.Tensor] = None, page_table: Optional[torch.Tensor] = None,
+                page_size: int = 0, pool_heads: int = 0, pool_hd: int = 0):
+    """For every (token, head): copy ``width`` features from src[t, src_off + h*src_head_stride ...], the first
+    ``rot_dims`` of them rotated by position (feature i pairs with i + rot_dims/2; angle = position *
+    inv_freq[i]; cos and sin times ``mag``), to rows of ``dst`` (ROTATE_TO_ROWS: dst[t, dst_off +
+    h*dst_head_stride ...]) or into the paged cache in the key or value layout, at feature dst_off of cached
+    head h (``pool_heads`` heads of ``pool_hd`` features a token)."""
+    ld_src = _ld(src, "rotate source")
+    n = src.shape[0]
+    if src_off < 0 or src_off + (heads - 1) * src_head_stride + width > src.shape[1]:
+        raise KernelError(f"rotate_copy: {heads} heads of {width} features from column {src_off} (stride "
+                          f"{src_head_stride}) do not fit rows of {src.shape[1]}")
+    _need(positions, "rotate positions", torch.int32, (n,))
+    if rot_dims:
+        _need(inv_freq, "rotate inv_freq", torch.float32, (rot_dims // 2,))
+    ld_dst, tw = 0, 0
+    if mode == ROTATE_TO_ROWS:
+        ld_dst = _ld(dst, "rotate destination")
+        if dst.shape[0] != n or dst_off < 0 or dst_off + (heads - 1) * dst_head_stride + width > dst.shape[1]:
+            raise KernelError(f"rotate_copy: {heads} heads of {width} features to column {dst_off} (stride "
+                              f"{dst_head_stride}) do not fit {tuple(dst.shape)}")
+    else:
+        _need(tok_slot, "rotate token slots", torch.int32, (n,))
+        _need(page_table, "rotate page table", torch.int32, (None, None))
+        _need(dst, "rotate pool", shape=(None, page_size, pool_heads * pool_hd))
+        tw = page_table.shape[1]
+    _check(_fn("attention_general", "cpmcu_rotate_copy")(
+        _p(src), c_int(_code(src)), c_long(ld_src), c_long(src_head_stride), c_long(src_off), _p(dst),
+        c_int(_code(dst)), c_int(mode), c_long(ld_dst), c_long(dst_head_stride), c_long(dst_off), c_int(n),
+        c_int(heads), c_int(width), c_int(rot_dims), _p(positions), _p(tok_slot), _p(inv_freq), c_float(mag),
+        _p(page_table), c_int(tw), c_int(page_size), c_int(pool_heads), c_int(pool_hd), _stream()))
+
+
+def attention_general(q: torch.Tensor, out: torch.Tensor, nh: int, nkv: int, hdk: int, hdv: int, scale: float,
+                      kpool: torch.Tensor, vpool: torch.Tensor, page_table: torch.Tensor, page_size: int,
+                      positions: torch.Tensor, tok_slot: torch.Tensor, chunk: int = 0):
+    """Causal attention with key size hdk and value size hdv of their own (plain kernel, both element types).
+    The cache may hold heads padded to a multiple of 16 features.  chunk > 0: the query at position p sees only
+    keys j <= p with j // chunk == p // chunk."""
+    _need(q, "attention q", shape=(None, nh * hdk))
+    n = q.shape[0]
+    _need(out, "attention out", q.dtype, (n, nh * hdv))
+    _need(kpool, "attention key pool", q.dtype, (None, page_size, None))
+    _need(vpool, "attention value pool", q.dtype, (kpool.shape[0], page_size, None))
+    if kpool.shape[2] % nkv or vpool.shape[2] % nkv:
+        raise KernelError(f"attention_general: pools of {kpool.shape[2]} / {vpool.shape[2]} features do not hold {nkv} heads")
+    _need(page_table, "attention page table", torch.int32, (None, None))
+    _need(positions, "attention positions", torch.int32, (n,))
+    _need(tok_slot, "attention token slots", torch.int32, (n,))
+    _check(_fn("attention_general", "cpmcu_attention_general")(
+        _p(q), _p(out), c_int(_code(q)), c_int(n), c_int(nh), c_int(nkv), c_int(hdk), c_int(hdv),
+        c_int(kpool.shape[2] // nkv), c_int(vpool.shape[2] // nkv), c_float(scale), c_int(chunk), _p(kpool),
+        _p(vpool), _p(page_table), c_int(page_table.shape[1]), c_int(page_size), _p(positions), _p(tok_slot),
+        _stream()))
+
+
+def gemm_heads(x: torch.Tensor, x_off: int, x_head_stride: int, w: torch.Tensor, out: torch.Tensor, out_off: int,
+               out_head_stride: int, gate: Optional[torch.Tensor] = None):
+    """out[m, out_off + h*out_head_stride + :N] = x[m, x_off + h*x_head_stride + :K] . w[h]^T for every head h;
+    w [H, N, K].  With ``gate`` [m, H] head h's rows are multiplied by sigmoid(gate[m, h])."""
+    ldx, ldy = _ld(x, "heads x"), _ld(out, "heads out")
+    M = x.shape[0]
+    _need(w, "heads weight", x.dtype, (None, None, None))
+    H, N, K = w.shape
+    if x_off < 0 or x_off + (H - 1) * x_head_stride + K > x.shape[1]:
+        raise KernelError(f"gemm_heads: {H} heads of {K} features from column {x_off} do not fit rows of {x.shape[1]}")
+    if out.shape[0] != M or out_off < 0 or out_off + (H - 1) * out_head_stride + N > out.shape[1]:
+        raise KernelError(f"gemm_heads: {H} heads of {N} features to column {out_off} do not fit {tuple(out.shape)}")
+    ldg = 0
+    if gate is not None:
+        ldg = _ld(gate, "heads gate")
+        if gate.dtype != x.dtype or tuple(gate.shape) != (M, H):
+            raise KernelError(f"heads gate: {gate.dtype} {tuple(gate.shape)}, expected {x.dtype} {(M, H)}")
+    xp = c_void_p(x.data_ptr() + x_off * x.element_size())
+    op = c_void_p(out.data_ptr() + out_off * out.element_size())
+    _check(_fn("gemm", "cpmcu_gemm_nt_heads")(xp, c_long(ldx), c_long(x_head_stride), _p(w), op, c_long(ldy),
+                                              c_long(out_head_stride), _p(gate), c_long(ldg), c_int(_code(x)),
+                                              c_int(_code(out)), c_int(M), c_int(H), c_int(N), c_int(K), _stream()))
+
+
 def argmax(logits: torch.Tensor, out: torch.Tensor):
     """out[r] = index of the largest logits[r] (ties: the lowest index)."""
     _need(logits, "argmax logits", torch.float32, (None, None))
@@ -757,3 +970,13 @@ def attention(q, out, nh, nkv, hd, scale, kpool, vpool, page_table, page_size, c
         return
     attention_plain(q, out, nh, nkv, hd, scale, kpool, vpool, page_table, page_size, ctx.positions, ctx.tok_slot,
                     sel_blocks, sel_count, block_size)
+
+
+def attention_any(q, out, nh, nkv, hdk, hdv, scale, kpool, vpool, page_table, page_size, ctx, chunk: int = 0):
+    """Attention with key and value sizes of their own and an optional chunked mask, with the kernel that suits
+    the step; writes ``out`` [n, nh*hdv]."""
+    if hdk == hdv and chunk == 0 and kpool.shape[2] == nkv * hdk:
+        attention(q, out, nh, nkv, hdk, scale, kpool, vpool, page_table, page_size, ctx)
+        return
+    attention_general(q, out, nh, nkv, hdk, hdv, scale, kpool, vpool, page_table, page_size, ctx.positions,
+                      ctx.tok_slot, chunk)

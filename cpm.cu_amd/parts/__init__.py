@@ -3,8 +3,10 @@ from .base import (BLOCKS, FEED_FORWARDS, MIXERS, NORMS, POSITION_ENCODINGS, Blo
                    PartSpec, PositionEncoding, Registry, ResidualStream, Runtime, StepContext, WeightSpec, Workspace)
 from .linear import Linear
 from .norm import RMSNorm
-from .rope import LongRotaryEncoding, RotaryEncoding
-from .attention import GQAAttention, InfLLMv2Attention
-from .ffn import GatedFFN
-from .block import PreNormBlock
+from .rope import LongRotaryEncoding, RotaryEncoding, YarnRotaryEncoding
+from .attention import GeneralAttention, GQAAttention, InfLLMv2Attention
+from .latent_attention import LatentAttention
+from .ssm import Mamba2Mixer
+from .ffn import GatedFFN, PolyNormFFN
+from .block import PreNormBlock, SandwichNormBlock
 from .embedding import LMHead, TokenEmbedding

@@ -214,3 +214,70 @@ class InfLLMv2Attention(GQAAttention):
                                   sel_blocks, sel_count, scratch=scratch)
             sel = (sel_blocks, sel_count, self.bs, self.window_blocks)
         return self.attend_and_project(q, ctx, cache, sel, defer_last=defer_last)
+
+
+def _pad16(n: int) -> int:
+    return -(-n // 16) * 16
+
+
+@MIXERS.register("attention")
+class GeneralAttention(Mixer):
+    """Grouped-query attention whose sizes are free: key size and value size of their own, a rotation that may
+    cover only the first features of a head (the rest pass unchanged), a score scale from the configuration,
+    and an optional chunked mask: the query at position p sees key j <= p only if j // chunk == p // chunk,
+    chunks counted from position 0 of the sequence (not from where a prompt was cut).  Query head h reads kv head
+    h // (heads / kv_heads); no biases; softmax in float.  With a chunked mask the cache keeps a trailing window
+    of one chunk and gives older pages back.  ``names``: checkpoint tensors for 'q', 'k', 'v', 'out'."""
+
+    def __init__(self, names: Mapping[str, str], hidden_size: int, num_heads: int, num_kv_heads: int, key_dim: int,
+                 value_dim: int, position: Optional[PositionEncoding], scale: float, mask_chunk: Optional[int] = None):
+        if num_heads % num_kv_heads:
+            raise ValueError(f"attention: {num_heads} heads are not a multiple of {num_kv_heads} kv heads")
+        if key_dim > 1024 or value_dim > 1024:
+            raise ValueError(f"attention: key size {key_dim} / value size {value_dim} exceed the kernel's 1024")
+        if mask_chunk is not None and mask_chunk <= 0:
+            raise ValueError(f"attention: a mask chunk of {mask_chunk} tokens")
+        self.names = dict(names)
+        self.hidden_size, self.nh, self.nkv, self.dk, self.dv = hidden_size, num_heads, num_kv_heads, key_dim, value_dim
+        self.position, self.scale, self.chunk = position, float(scale), int(mask_chunk or 0)
+        self.qkv = Linear([(self.names["q"], num_heads * key_dim), (self.names["k"], num_kv_heads * key_dim),
+                           (self.names["v"], num_kv_heads * value_dim)], hidden_size)
+        self.o = Linear([(self.names["out"], hidden_size)], num_heads * value_dim)
+
+    def parts(self) -> List[Part]:
+        return [self.qkv, self.o] + ([self.position] if self.position is not None else [])
+
+    def bind(self, tensors: Mapping[str, torch.Tensor], rt: Runtime):
+        self.rt = rt
+
+    def cache_needs(self) -> CacheNeeds:
+        return CacheNeeds(streams=(("k", StreamSpec(self.nkv * _pad16(self.dk))),
+                                   ("v", StreamSpec(self.nkv * _pad16(self.dv)))),
+                          window=self.chunk or None)
+
+    def forward(self, h, ctx: StepContext, cache: CacheView, writes_cache: bool = True):
+        n, nh, nkv, dk, dv = h.shape[0], self.nh, self.nkv, self.dk, self.dv
+        rot = self.position.rotary_params() if self.position is not None else None
+        if self.position is not None and rot is None:
+            raise ValueError("attention: the position encoding must be a rotation (rotary_params)")
+        inv_freq, mag = rot if rot is not None else (None, 1.0)
+        rd = 0 if inv_freq is None else 2 * inv_freq.shape[0]
+        if rd > dk:
+            raise ValueError(f"attention: the rotation covers {rd} features, a head has {dk}")
+        with ctx.timed("attn_qkv_rope"):
+            qkv = self.qkv.forward(h, ctx, "attn.qkv", rows=None if writes_cache else nh * dk)
+            q = ctx.ws.get("attn.q", (n, nh * dk), self.rt.dtype)
+            ops.rotate_copy(qkv, 0, dk, nh, dk, rd, ctx.positions, inv_freq, mag, q, ops.ROTATE_TO_ROWS, 0, dk)
+            if writes_cache:
+                kp, vp = cache.streams["k"], cache.streams["v"]
+                paged = dict(tok_slot=ctx.tok_slot, page_table=cache.page_table, page_size=cache.page_size, pool_heads=nkv)
+                ops.rotate_copy(qkv, nh * dk, dk, nkv, dk, rd, ctx.positions, inv_freq, mag, kp, ops.ROTATE_TO_KEYS,
+                                pool_hd=kp.shape[2] // nkv, **paged)
+                ops.rotate_copy(qkv, (nh + nkv) * dk, dv, nkv, dv, 0, ctx.positions, None, 1.0, vp,
+                                ops.ROTATE_TO_VALUES, pool_hd=vp.shape[2] // nkv, **paged)
+        out = ctx.ws.get("attn.out", (n, nh * dv), self.rt.dtype)
+        with ctx.timed("attn_core"):
+            ops.attention_any(q, out, nh, nkv, dk, dv, self.scale, cache.streams["k"], cache.streams["v"],
+                              cache.page_table, cache.page_size, ctx, chunk=self.chunk)
+        with ctx.timed("attn_o"):
+            return self.o.forward(out, ctx, "attn.o", out_dtype=torch.float32, partials=True)

@@ -17,6 +17,8 @@ Kinds of parts and what each must provide:
 * ``Block``:     forward(stream, ctx, cache, writes_cache): the arrangement of the above
                  around the residual stream
 
+A branch may have a norm of its own before it joins the residual (``NormedBranch``; ``Norm.normalize``).
+
 Two optional protocols let neighbouring parts share a kernel without knowing each other: a norm may leave
 its row factor to the product that follows (``forward_unscaled`` / ``takes_row_scale``), and a part may leave
 its last product to the norm that follows (``DeferredBranch``: ``can_defer_last`` /
@@ -152,9 +154,35 @@ class DeferredBranch:
         return self._value
 
 
+class NormedBranch:
+    """A branch that passes a norm of its own before it joins the residual: x += ``norm``(``branch``) (the
+    arrangement with a norm before and after every sub-layer).  A norm that knows a kernel which does this
+    together with its own work takes it as it is (``Norm.takes_normed_branch``); for everybody else
+    ``evaluate()`` runs ``norm.normalize`` and gives the tensor to add."""
+
+    def __init__(self, branch, norm: "Norm", ctx: "StepContext", tag: str):
+        self.branch, self.norm, self.ctx, self.tag = branch, norm, ctx, tag
+        self._value: Optional[torch.Tensor] = None
+
+    def evaluate(self) -> torch.Tensor:
+        if self._value is None:
+            self._value = self.norm.normalize(branch_tensor(self.branch), self.ctx, self.tag)
+        return self._value
+
+
 def branch_tensor(branch):
     """The branch as a tensor (or None), whatever form it was handed over in."""
-    return branch.evaluate() if isinstance(branch, DeferredBranch) else branch
+    return branch.evaluate() if isinstance(branch, (DeferredBranch, NormedBranch)) else branch
+
+
+def branch_for(norm: "Norm", branch):
+    """The branch in a form that ``norm.forward`` accepts: as it is if the norm declares that it takes that
+    form, else as a tensor."""
+    if isinstance(branch, DeferredBranch) and not norm.takes_deferred_branch:
+        return branch.evaluate()
+    if isinstance(branch, NormedBranch) and not norm.takes_normed_branch:
+        return branch.evaluate()
+    return branch
 
 
 class ResidualStream:
@@ -239,6 +267,13 @@ class Norm(Part):
 
     # True if forward and forward_unscaled accept a DeferredBranch as ``branch``
     takes_deferred_branch = False
+    # True if forward and forward_unscaled accept a NormedBranch as ``branch``
+    takes_normed_branch = False
+
+    def normalize(self, t: torch.Tensor, ctx: StepContext, tag: str = "norm.plain") -> torch.Tensor:
+        """The norm of the rows of ``t`` alone, float32 [n, H]: no residual, nothing added (what a branch that
+        has a norm of its own passes through, NormedBranch)."""
+        raise NotImplementedError
 
 
 class PositionEncoding(Part):

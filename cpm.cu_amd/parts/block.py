@@ -11,8 +11,8 @@ from __future__ import annotations
 from typing import List, Optional
 
 from ..cache.paged import CacheView
-from .base import (BLOCKS, Block, DeferredBranch, FeedForward, Mixer, Norm, Part, ResidualStream, StepContext, branch_tensor,
-                   forward_declares)
+from .base import (BLOCKS, Block, DeferredBranch, FeedForward, Mixer, Norm, NormedBranch, Part, ResidualStream,
+                   StepContext, branch_for, forward_declares)
 
 
 @BLOCKS.register("pre_norm")
@@ -37,8 +37,7 @@ class PreNormBlock(Block):
     def _normed(norm: Norm, deferred: bool, x, branch, branch_scale, ctx):
         """The normed rows and None, or (if the consumer finishes the norm itself) the rows without the norm's
         row factor and that factor's ingredients."""
-        if not norm.takes_deferred_branch:
-            branch = branch_tensor(branch)
+        branch = branch_for(norm, branch)
         # a norm that takes a branch's last product over runs it in the same kernel: the label says so
         label = "norm+" + branch.tag.split(".")[-1] if isinstance(branch, DeferredBranch) else "norm"
         with ctx.timed(label):
@@ -74,3 +73,38 @@ class PreNormBlock(Block):
         with ctx.timed("ffn"):
             stream.pending = self._feed(stream, a, ctx)
         stream.pending_scale = self.residual_scale
+
+
+@BLOCKS.register("sandwich_norm")
+class SandwichNormBlock(Block):
+    """A norm before and after every sub-layer: x += post1(Mixer(norm1(x))); x += post2(FeedForward(norm2(x))).
+    A layer may have no feed-forward.  The branch with its post-norm is left pending (NormedBranch) for the
+    norm that follows, which adds it into the residual while it norms the sum."""
+
+    def __init__(self, mixer_norm: Norm, mixer: Mixer, mixer_post_norm: Norm, ff_norm: Optional[Norm] = None,
+                 feed_forward: Optional[FeedForward] = None, ff_post_norm: Optional[Norm] = None):
+        if (feed_forward is None) != (ff_norm is None) or (feed_forward is None) != (ff_post_norm is None):
+            raise ValueError("sandwich_norm: a feed-forward comes with both of its norms, or none of the three is given")
+        self.mixer_norm, self.mixer, self.mixer_post_norm = mixer_norm, mixer, mixer_post_norm
+        self.ff_norm, self.feed_forward, self.ff_post_norm = ff_norm, feed_forward, ff_post_norm
+
+    def parts(self) -> List[Part]:
+        out = [self.mixer_norm, self.mixer, self.mixer_post_norm]
+        if self.feed_forward is not None:
+            out += [self.ff_norm, self.feed_forward, self.ff_post_norm]
+        return out
+
+    def forward(self, stream: ResidualStream, ctx: StepContext, cache: Optional[CacheView], writes_cache: bool = True):
+        with ctx.timed("attn"):
+            with ctx.timed("norm"):
+                h = self.mixer_norm.forward(stream.x, branch_for(self.mixer_norm, stream.take_pending()),
+                                            stream.pending_scale, ctx, tag="block.h")
+            a = NormedBranch(self.mixer.forward(h, ctx, cache, writes_cache), self.mixer_post_norm, ctx, "block.post")
+        if self.feed_forward is None:
+            stream.pending = a
+        else:
+            with ctx.timed("ffn"):
+                with ctx.timed("norm"):
+                    h = self.ff_norm.forward(stream.x, branch_for(self.ff_norm, a), 1.0, ctx, tag="block.h")
+                stream.pending = NormedBranch(self.feed_forward.forward(h, ctx), self.ff_post_norm, ctx, "block.post")
+        stream.pending_scale = 1.0

@@ -5,12 +5,12 @@ gate and up are one stacked product, gate rows first (src/model/ffn.cuh:31-59,
 """
 from __future__ import annotations
 
-from typing import List
+from typing import List, Mapping
 
 import torch
 
 from .. import ops
-from .base import FEED_FORWARDS, DeferredBranch, FeedForward, Part, StepContext
+from .base import FEED_FORWARDS, DeferredBranch, FeedForward, Part, Runtime, StepContext, WeightSpec
 from .linear import Linear
 
 
@@ -36,5 +36,37 @@ class GatedFFN(FeedForward):
             act = self.gate_up.forward_gated(h, ctx, "ffn.gate_up", row_scale=row_scale)
         if defer_last and self.down.defers(act):
             return DeferredBranch(self.down, act, ctx, "ffn.down")
+        with ctx.timed("ffn_down"):
+            return self.down.forward(act, ctx, "ffn.down", out_dtype=torch.float32, partials=True)
+
+
+@FEED_FORWARDS.register("poly_norm")
+class PolyNormFFN(FeedForward):
+    """down( act(up x) ) with the PolyNorm activation act(z) = a N(z) + b N(z^2) + c N(z^3) + e: powers element by
+    element, N divides a token's vector by its root mean square sqrt(mean(v^2) + eps); the four numbers are a
+    checkpoint tensor.  The statistics and the polynomial are computed in float."""
+
+    def __init__(self, up_name: str, down_name: str, act_name: str, hidden_size: int, intermediate_size: int, eps: float):
+        self.hidden_size, self.intermediate_size, self.eps = hidden_size, intermediate_size, float(eps)
+        self.act_name = act_name
+        self.up = Linear([(up_name, intermediate_size)], hidden_size)
+        self.down = Linear([(down_name, hidden_size)], intermediate_size)
+
+    def parts(self) -> List[Part]:
+        return [self.up, self.down]
+
+    def weight_specs(self) -> List[WeightSpec]:
+        return [WeightSpec(self.act_name, (4,), "poly_coefficients")]
+
+    def bind(self, tensors: Mapping[str, torch.Tensor], rt: Runtime):
+        self.coef = tensors[self.act_name].to(torch.float32).contiguous()
+        self.rt = rt
+
+    def forward(self, h: torch.Tensor, ctx: StepContext):
+        with ctx.timed("ffn_up"):
+            z = self.up.forward(h, ctx, "ffn.up", partials=True)
+        act = ctx.ws.get("ffn.act", (h.shape[0], self.intermediate_size), self.rt.dtype)
+        with ctx.timed("ffn_act"):
+            ops.poly_norm(z, self.coef, self.eps, act)
         with ctx.timed("ffn_down"):
             return self.down.forward(act, ctx, "ffn.down", out_dtype=torch.float32, partials=True)

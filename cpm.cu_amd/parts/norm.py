@@ -11,29 +11,46 @@ from typing import List, Mapping, Optional
 import torch
 
 from .. import ops
-from .base import NORMS, DeferredBranch, Norm, Runtime, StepContext, WeightSpec, branch_tensor
+from .base import NORMS, DeferredBranch, Norm, NormedBranch, Runtime, StepContext, WeightSpec, branch_tensor
 
 
 @NORMS.register("rms_norm")
 class RMSNorm(Norm):
-    def __init__(self, name: str, hidden_size: int, eps: float):
+    """``unit_offset``: the checkpoint stores the weight around zero and the norm multiplies by 1 + w."""
+
+    def __init__(self, name: str, hidden_size: int, eps: float, unit_offset: bool = False):
         self.name = name
         self.hidden_size = hidden_size
         self.eps = float(eps)
+        self.unit_offset = bool(unit_offset)
 
     def weight_specs(self) -> List[WeightSpec]:
-        return [WeightSpec(self.name, (self.hidden_size,), "norm")]
+        return [WeightSpec(self.name, (self.hidden_size,), "norm_offset" if self.unit_offset else "norm")]
 
     def bind(self, tensors: Mapping[str, torch.Tensor], rt: Runtime):
-        self.weight = tensors[self.name].to(torch.float32).contiguous()
+        w = tensors[self.name].to(torch.float32)
+        self.weight = (w + 1.0 if self.unit_offset else w).contiguous()
         self.rt = rt
 
     takes_deferred_branch = True
+    takes_normed_branch = True
+
+    def normalize(self, t, ctx: StepContext, tag="norm.plain"):
+        if t.dim() == 3:                       # float partial sums of a split product
+            t = t.sum(0) if t.shape[0] > 1 else t[0]
+        out = ctx.ws.get(tag, (t.shape[0], self.hidden_size), torch.float32)
+        ops.rms_norm_groups(t, self.weight, self.eps, out)
+        return out
 
     def forward(self, x, branch, branch_scale, ctx: StepContext, rows=None, tag="norm"):
-        branch = branch_tensor(branch)
         n_out = x.shape[0] if rows is None else rows.shape[0]
         out = ctx.ws.get(tag, (n_out, self.hidden_size), self.rt.dtype)
+        if isinstance(branch, NormedBranch) and isinstance(branch.norm, RMSNorm) and branch_scale == 1.0:
+            # the branch's own norm, the residual add and this norm in one pass over the row
+            ops.branch_norm_add_norm(x, branch_tensor(branch.branch), branch.norm.weight, branch.norm.eps,
+                                     self.weight, self.eps, out, rows)
+            return out
+        branch = branch_tensor(branch)
         ops.add_rms_norm(x, branch, branch_scale, self.weight, self.eps, out, rows)
         return out
 
@@ -41,6 +58,8 @@ class RMSNorm(Norm):
         # decode steps: a row a workgroup leaves most of the chip idle, so the work is cut by columns and the
         # row factor rsqrt(mean(x^2) + eps) is left to the product that follows
         n = x.shape[0]
+        if isinstance(branch, NormedBranch):
+            return None
         if self.rt.dtype != torch.bfloat16 or not ops.strip_kernels_ok(n, self.hidden_size) or self.hidden_size % 4:
             return None
         out = ctx.ws.get(tag, (n, self.hidden_size), torch.bfloat16)

@@ -59,3 +59,30 @@ class LongRotaryEncoding(RotaryEncoding):
 
     def factors(self, max_seq_len: int):
         return self.long_factor if max_seq_len > self.original_max_position else self.short_factor
+
+
+@POSITION_ENCODINGS.register("yarn")
+class YarnRotaryEncoding(RotaryEncoding):
+    """Rotation of ``head_dim`` features (a head may hold more; those pass unchanged) with YaRN's blend of
+    stretched and plain frequencies.  With f_i = theta^(-2i/head_dim):
+        d(t)   = head_dim * ln(original / (2 pi t)) / (2 ln theta)        (the feature that turns t times)
+        lo, hi = max(floor(d(fast)), 0), min(ceil(d(slow)), head_dim - 1)
+        ramp_i = clamp((i - lo) / max(hi - lo, 0.001), 0, 1)
+        freq_i = f_i / factor * ramp_i + f_i * (1 - ramp_i)
+    and cos and sin carry the magnitude 0.1 ln(factor) + 1."""
+
+    def __init__(self, head_dim: int, theta: float, factor: float, original: int, fast: float, slow: float):
+        super().__init__(head_dim, theta)
+        self.factor, self.original, self.fast, self.slow = float(factor), float(original), float(fast), float(slow)
+        self.magnitude = 0.1 * math.log(self.factor) + 1.0
+
+    def _turns_to_feature(self, turns: float) -> float:
+        return self.head_dim * math.log(self.original / (2.0 * math.pi * turns)) / (2.0 * math.log(self.theta))
+
+    def bind(self, tensors: Mapping[str, torch.Tensor], rt: Runtime):
+        i = torch.arange(0, self.head_dim // 2, dtype=torch.float64)
+        f = self.theta ** (-2.0 * i / self.head_dim)
+        lo = max(math.floor(self._turns_to_feature(self.fast)), 0)
+        hi = min(math.ceil(self._turns_to_feature(self.slow)), self.head_dim - 1)
+        ramp = ((i - lo) / max(hi - lo, 0.001)).clamp(0.0, 1.0)
+        self.inv_freq = (f / self.factor * ramp + f * (1.0 - ramp)).to(torch.float32).to(rt.device)

@@ -52,6 +52,42 @@ def _init_norm(spec, g, device, dtype, std, norm_std):
     return t.to(dtype)
 
 
+@register_init_rule("norm_offset")
+def _init_norm_offset(spec, g, device, dtype, std, norm_std):
+    """N(0, norm_std): the weight of a norm that multiplies by 1 + w."""
+    t = torch.zeros(spec.shape, dtype=torch.float32, device=device)
+    if norm_std > 0:
+        t += torch.randn(spec.shape, generator=g, dtype=torch.float32, device=device) * norm_std
+    return t.to(dtype)
+
+
+@register_init_rule("poly_coefficients")
+def _init_poly_coefficients(spec, g, device, dtype, std, norm_std):
+    """The numbers of a polynomial activation: each of order 1, none near zero, signs mixed."""
+    t = 0.4 + torch.rand(spec.shape, generator=g, dtype=torch.float32, device=device)
+    sign = torch.where(torch.rand(spec.shape, generator=g, dtype=torch.float32, device=device) < 0.3, -1.0, 1.0)
+    return (t * sign).to(dtype)
+
+
+@register_init_rule("small")
+def _init_small(spec, g, device, dtype, std, norm_std):
+    """N(0, 0.5): biases of a convolution or of a step size."""
+    return (torch.randn(spec.shape, generator=g, dtype=torch.float32, device=device) * 0.5).to(dtype)
+
+
+@register_init_rule("conv_taps")
+def _init_conv_taps(spec, g, device, dtype, std, norm_std):
+    """N(0, 1/sqrt(taps)): the taps of a short convolution per channel."""
+    return (torch.randn(spec.shape, generator=g, dtype=torch.float32, device=device) * spec.shape[-1] ** -0.5).to(dtype)
+
+
+@register_init_rule("log_decay")
+def _init_log_decay(spec, g, device, dtype, std, norm_std):
+    """ln of decay rates spread over (0.05, 4): slow heads that remember far back and fast ones."""
+    u = torch.rand(spec.shape, generator=g, dtype=torch.float32, device=device)
+    return torch.log(0.05 + 3.95 * u).to(dtype)
+
+
 @register_init_rule("matrix")
 def _init_matrix(spec, g, device, dtype, std, norm_std):
     """N(0, std)."""
