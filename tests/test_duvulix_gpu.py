@@ -1,0 +1,205 @@
+"""The Duvulix engine against the plain implementation (GPU): whole prompts, prefill against token-by-token
+decoding, portions of several sizes down to two tokens, unequal batches against each request alone, slots and
+pages that are used again, long decoding across chunk and page edges, the first tokens of a sequence, and
+greedy generation through the package's own entry point and scheduler."""
+import pytest
+import torch
+
+import plain_duvulix as plain
+import schedules
+import tiny
+import tiny_duvulix as td
+
+pytestmark = pytest.mark.gpu
+
+# P: chunk of 40, pages of 64; Q: chunk of 33.  Lengths cross several chunks and pages.
+LENS = {"a": 13, "b": 171, "c": 85, "d": 41, "e": 1, "f": 2}
+PROMPT = {"a": 5, "b": 130, "c": 64, "d": 39, "e": 1, "f": 1}
+BATCHES = [("a", "b", "c"), ("d", "e", "f"), ("c", "a"), ("f", "b", "d")]
+
+
+@pytest.fixture(scope="module")
+def models(tmp_path_factory):
+    out = {}
+    for name, raw, seed in (("P", td.tiny_p(), 31), ("Q", td.tiny_q(), 47)):
+        d = str(tmp_path_factory.mktemp(f"duvulix_{name}"))
+        td.write_model(raw, d, seed)
+        cfg, w = tiny.read_model(d)
+        reqs = {r: tiny.random_tokens(n, raw["vocab"], 500 + i) for i, (r, n) in enumerate(LENS.items())}
+        out[name] = (d, cfg, w, reqs, {r: plain.forward(cfg, w, t).float() for r, t in reqs.items()})
+    return out
+
+
+_engines = {}
+
+
+def engine_for(models, name, dtype, **kw):
+    from cpmcu_amd import Engine, EngineOptions
+    key = (name, dtype, tuple(sorted(kw.items())))
+    if key not in _engines:
+        opts = dict(dtype=dtype, max_tokens=1024, max_slots=3, max_seq_len=512)
+        opts.update(kw)
+        _engines[key] = Engine.from_dir(models[name][0], EngineOptions(**opts))
+    return _engines[key]
+
+
+def check(got, refs, dtype, what):
+    """float32 (the sharp comparison): rounding of float sums on logits of size ~1, at every position.
+    bfloat16: the deviation of a position's logits (mean taken off) against the logits' spread: 0.05 at
+    most, with up to one position in fifty of a request (or one) beyond that but within 0.25.  Such positions
+    exist by the design and not by the kernels: where a token's gated values of one norm group are all nearly
+    zero, the group's norm magnifies the rounding of the projection before it (the plain implementation with its
+    own projections rounded to bfloat16 shows the same positions)."""
+    for r, ref in refs.items():
+        if dtype == "float32":
+            err = (got[r] - ref).abs().max(dim=1).values
+            bad = (err > 1e-4).nonzero().flatten()
+            assert bad.numel() == 0, (f"{what}: request {r}: first wrong position {int(bad[0])} of {ref.shape[0]} "
+                                      f"(error {float(err[bad[0]]):.3g})")
+            continue
+        d = got[r] - ref
+        err = (d - d.mean(1, keepdim=True)).pow(2).mean(1).sqrt() / ref.std()
+        over = (err > 0.05).nonzero().flatten()
+        assert over.numel() <= max(1, ref.shape[0] // 50) and float(err.max()) <= 0.25 and float(err.median()) <= 0.02, \
+            (f"{what}: request {r}: {over.numel()} of {ref.shape[0]} positions over 0.05 (first {int(over[0]) if over.numel() else -1}, "
+             f"worst {float(err.max()):.3g}, median {float(err.median()):.3g})")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["P", "Q"])
+def test_whole_prompts(models, name, dtype):
+    _, cfg, w, reqs, refs = models[name]
+    eng = engine_for(models, name, dtype)
+    check(schedules.whole(eng, reqs), refs, dtype, "whole")
+    eng.cache.check()
+    assert not eng.cache.live
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["P", "Q"])
+def test_prefill_then_token_by_token(models, name, dtype):
+    _, cfg, w, reqs, refs = models[name]
+    eng = engine_for(models, name, dtype)
+    check(schedules.tail(eng, reqs, 45), refs, dtype, "tail-45")       # 45 tokens cross a chunk's edge in decoding
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["P", "Q"])
+def test_unequal_batches_and_slots_used_again(models, name, dtype):
+    _, cfg, w, reqs, refs = models[name]
+    eng = engine_for(models, name, dtype)
+    for part in (BATCHES[:2], BATCHES[2:]):
+        used = {r for b in part for r in b}
+        got = schedules.batched(eng, {r: reqs[r] for r in used}, PROMPT, part)
+        check(got, {r: refs[r] for r in used}, dtype, "batched")
+    eng.cache.check()
+    assert not eng.cache.live
+
+
+@pytest.mark.parametrize("step", [2, 7, 33, 64])
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["P", "Q"])
+def test_portions(models, name, dtype, step):
+    """Forward passes of at most `step` tokens: a prompt is cut into portions, and a batch's sequences are
+    split across passes."""
+    _, cfg, w, reqs, refs = models[name]
+    eng = engine_for(models, name, dtype, max_step_tokens=step)
+    some = {r: reqs[r] for r in ("b", "d", "f")}
+    check(schedules.whole(eng, some), {r: refs[r] for r in some}, dtype, f"portions of {step}")
+    got = schedules.batched(eng, {r: reqs[r] for r in ("c", "a", "d")}, PROMPT, [("c", "a", "d")])
+    check(got, {r: refs[r] for r in ("c", "a", "d")}, dtype, f"batch in portions of {step}")
+    eng.cache.check()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["P", "Q"])
+def test_long_decoding_from_the_first_token(models, name, dtype):
+    """One token, then 170 more one by one (captured graphs): every chunk edge and two page edges are crossed
+    in decoding, and the state of the recurrent layers is carried all the way."""
+    _, cfg, w, reqs, refs = models[name]
+    eng = engine_for(models, name, dtype, hip_graph=True)
+    got = schedules.tail(eng, {"b": reqs["b"]}, len(reqs["b"]) - 1)
+    check(got, {"b": refs["b"]}, dtype, "decoding from the first token")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_request_does_not_depend_on_its_neighbours_or_its_pages(models, dtype):
+    """The same request alone, in a batch of unequal requests, and again after other requests have used and
+    freed the slots and pages: the same logits beyond rounding."""
+    from cpmcu_amd import StepEntry
+    _, cfg, w, reqs, refs = models["P"]
+    eng = engine_for(models, "P", dtype)
+    alone = schedules.whole(eng, {"c": reqs["c"]})["c"]
+    s = [eng.acquire() for _ in range(3)]
+    b_len = 0
+    lg = eng.step([StepEntry(s[0], reqs["b"], []), StepEntry(s[1], reqs["c"], list(range(LENS["c"]))),
+                   StepEntry(s[2], reqs["a"], [0])]).cpu()
+    for x in (s[1], s[0], s[2]):
+        eng.release(x)
+    again = schedules.whole(eng, {"c": reqs["c"]})["c"]
+    # alone and again run the same kernels on the same rows: equal bit for bit; in the batch the products take
+    # other numbers of rows, which changes the order of their sums
+    assert torch.equal(again, alone)
+    if dtype == "float32":
+        assert float((lg[b_len:b_len + LENS["c"]] - alone).abs().max()) <= 2e-5
+    else:
+        check({"c": lg[b_len:b_len + LENS["c"]]}, {"c": alone}, dtype, "in a batch against alone")
+
+
+def test_residual_stream_layer_by_layer(models):
+    """float32: the residual after every layer equals the plain implementation's (the branch a layer leaves
+    pending is added by the next norm, so the stream is read after the following layer's first norm ran)."""
+    from cpmcu_amd import StepEntry
+    _, cfg, w, reqs, refs = models["P"]
+    eng = engine_for(models, "P", "float32")
+    res = []
+    plain.forward(cfg, w, reqs["d"], res)
+    seen = []
+    blocks = eng.model.layers
+    originals = [b.mixer_norm.forward for b in blocks]
+
+    def spy(i):
+        def f(x, *a, **k):
+            out = originals[i](x, *a, **k)
+            seen.append(x.clone())
+            return out
+        return f
+    try:
+        for i, b in enumerate(blocks):
+            b.mixer_norm.forward = spy(i)
+        s = eng.acquire()
+        eng.step([StepEntry(s, reqs["d"], [0])])
+        eng.release(s)
+    finally:
+        for b, o in zip(blocks, originals):
+            b.mixer_norm.forward = o
+    assert len(seen) == len(blocks)
+    for i in range(1, len(blocks)):
+        err = float((seen[i].cpu().double() - res[i - 1]).abs().max())
+        assert err < 5e-5, f"residual after layer {i - 1}: {err:.3g}"
+
+
+def test_greedy_generation_through_the_entry_point(models):
+    from cpmcu_amd.llm import LLM
+    d, cfg, w, reqs, refs = models["Q"]
+    prompt = reqs["a"][:9]
+    want = plain.greedy(cfg, w, prompt, 20)
+    llm = LLM(d, dtype="float32", max_tokens=256)
+    llm.init_storage()
+    llm.load_from_hf()
+    tokens, _, _ = llm.generate(torch.tensor(prompt, dtype=torch.int32), 20)
+    assert tokens == want
+
+
+def test_generation_loop_with_unequal_requests(models):
+    """The scheduler's own loop: several prompts of unequal length in batches, greedy, against the plain
+    implementation's tokens (float32)."""
+    from cpmcu_amd.engine.generate import generate
+    d, cfg, w, reqs, refs = models["P"]
+    eng = engine_for(models, "P", "float32")
+    prompts = [reqs["a"][:7], reqs["c"][:50], reqs["d"][:3], reqs["b"][:90]]
+    out = generate(eng, prompts, 12)                               # 3 slots: two batches, slots used again
+    for p, o in zip(prompts, out):
+        assert list(o.tokens) == plain.greedy(cfg, w, p, 12)
+    eng.cache.check()
+    assert not eng.cache.live
