@@ -172,10 +172,12 @@ def main():
     ap.add_argument("--perf", action="store_true",
                     help="after the timed runs, a few eager steps with the engine's timers on: average ms by kernel "
                          "class (products / attention / selection / norms / head) on stderr and under 'timers'")
-    ap.add_argument("--scenario", default="headline", choices=["headline", "small_batch64", "sparse32k"],
+    ap.add_argument("--scenario", default="headline", choices=["headline", "small_batch64", "sparse32k", "duvulix"],
                     help="headline: the 8B shape at batch 8, context 4,096 (the default, the contract's line); "
                          "small_batch64: the 0.5B shape, 64 unequal prompts through the generation loop; sparse32k: "
-                         "the 8B shape with InfLLM-v2 at 32k context")
+                         "the 8B shape with InfLLM-v2 at 32k context; duvulix: four Duvulix layers of a real model's "
+                         "sizes (latent attention, chunked attention, Mamba-2, a layer that reads the first one's "
+                         "latent cache) beside four MiniCPM4-8B layers of equal width: decode and prefill of both")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported (no multi-GPU path exists)")
@@ -358,8 +360,177 @@ def main():
     print(json.dumps(rec), flush=True)
 
 
+def config_duvulix():
+    """Four layers of sizes that resemble a real model's: width 4,096; latent attention with 32 heads of 128 + 64
+    features over a latent of 512; attention with 32 heads on 8 kv heads of 128, chunks of 2,048 tokens, YaRN;
+    Mamba-2 with 128 heads of 64, state 128, 8 groups; PolyNorm feed-forwards of 16,384."""
+    latent = {"heads": 32, "dim": 128, "rot_dim": 64, "vdim": 128, "kv_rank": 512, "scale": 192 ** -0.5,
+              "rot": {"base": 500000.0, "dims": 64}}
+    mlp = {"kind": "dense", "ff": 16384}
+    return {
+        "architecture": "Duvulix", "vocab": 73448, "width": 4096, "norm": {"eps": 1e-6},
+        "layers": [
+            {"type": "latent_attention", "mixer": dict(latent), "mlp": mlp},
+            {"type": "attention", "mixer": {"heads": 32, "kv_heads": 8, "dim": 128, "vdim": 128, "scale": 128 ** -0.5,
+                                            "rot": {"base": 500000.0, "dims": 128,
+                                                    "scaling": {"factor": 8.0, "original": 8192, "fast": 32.0, "slow": 1.0}},
+                                            "mask": {"size": 2048}}, "mlp": mlp},
+            {"type": "mamba2", "mixer": {"heads": 128, "vdim": 64, "state": 128, "groups": 8, "conv": 4,
+                                         "norm_groups": 8}, "mlp": mlp},
+            {"type": "latent_attention", "mixer": dict(latent, kv_from=0), "mlp": mlp},
+        ],
+    }
+
+
+def duvulix_step_bytes(raw, esize, batch, context):
+    """Bytes a decode step must move: every matrix once (the embedding's rows aside), and per sequence what its
+    mixers read: the latent cache once per layer that reads it, the keys and values of the query's chunk, the
+    recurrent state read and written."""
+    W = raw["width"]
+    weights = raw["vocab"] * W
+    per_seq = 0
+    for layer in raw["layers"]:
+        m = layer["mixer"]
+        if layer["type"] == "latent_attention":
+            weights += m["heads"] * (m["dim"] + m["rot_dim"]) * W + m["heads"] * W + m["heads"] * m["vdim"] * W
+            weights += m["heads"] * (m["dim"] + m["vdim"]) * m["kv_rank"]
+            if m.get("kv_from") is None:
+                weights += (m["kv_rank"] + m["rot_dim"]) * W
+            per_seq += context * (2 * m["kv_rank"] + m["rot_dim"]) * esize
+        elif layer["type"] == "attention":
+            weights += (m["heads"] * (m["dim"] + m["vdim"]) + m["kv_heads"] * (m["dim"] + m["vdim"])) * W
+            seen = context if not m.get("mask") else (context - 1) % m["mask"]["size"] + 1
+            per_seq += seen * m["kv_heads"] * (m["dim"] + m["vdim"]) * esize
+        else:
+            inner, gn = m["heads"] * m["vdim"], m["groups"] * m["state"]
+            weights += (2 * inner + 2 * gn + m["heads"]) * W + inner * W
+            per_seq += 2 * 4 * (m["heads"] * m["vdim"] * m["state"] + (m["conv"] - 1) * (inner + 2 * gn))
+        if layer.get("mlp"):
+            weights += 2 * layer["mlp"]["ff"] * W
+    return weights * esize + batch * per_seq, weights
+
+
+def duvulix_scenario(args, dev):
+    """Decode and prefill of the Duvulix layer shapes beside the MiniCPM4-8B layer shape (equal width, equal
+    number of layers, random weights): one JSON line with both models' figures and their timers by kernel class."""
+    import torch
+    import cpmcu_amd
+    from cpmcu_amd import Engine, EngineOptions, StepEntry, ops
+    from cpmcu_amd.weights import random_tensors
+
+    esize = 2 if args.dtype == "bfloat16" else 4
+    batches = sorted({1, args.batch, 32})
+    n_prefill = args.prefill_tokens
+    g = torch.Generator().manual_seed(7)
+    next_tok = torch.zeros(64, dtype=torch.int32, device=dev)
+    read_gbs = calibrate_read(dev)
+    out = {}
+    for name, raw in (("duvulix", config_duvulix()), ("minicpm", config_8b(4))):
+        arch = cpmcu_amd.get_architecture(raw.get("architecture") or raw["architectures"][0])
+        cfg = arch.config_class.from_dict(raw)
+        per_seq = -(-(args.context + args.steps + args.warmup + 64) // 64) * 64
+        eng = Engine.from_tensors(cfg, random_tensors(cfg, seed=0, device=dev), EngineOptions(
+            dtype=args.dtype, max_tokens=max(max(batches) * per_seq, n_prefill + 64), max_slots=max(batches),
+            max_seq_len=max(per_seq, n_prefill + 64), max_step_tokens=max(n_prefill, 2048), device=dev,
+            hip_graph=bool(args.hip_graph), rehearse=not args.no_rehearse))
+        rand_ids = lambda n: [int(t) for t in torch.randint(0, cfg.vocabulary_size, (n,), generator=g)]
+
+        def filled(batch):
+            slots = [eng.acquire() for _ in range(batch)]
+            for s in slots:
+                eng.cache.extend(s, args.context - 1)
+            eng.cache.sync()
+            for grp in eng.cache.groups:
+                for st in list(grp.storage.values()) + list(grp.state.values()):
+                    for t in st.values():
+                        t.normal_(0.0, 0.5)
+            return slots
+
+        def decode(batch, steps, warmup):
+            slots = filled(batch)
+            toks = [rand_ids(batch) for _ in range(steps + warmup)]
+            for i in range(warmup):
+                ops.argmax(eng.step([StepEntry(s, [toks[i][j]], [0]) for j, s in enumerate(slots)]), next_tok[:batch])
+            torch.cuda.synchronize()
+            t = time.perf_counter()
+            for i in range(warmup, warmup + steps):
+                ops.argmax(eng.step([StepEntry(s, [toks[i][j]], [0]) for j, s in enumerate(slots)]), next_tok[:batch])
+            torch.cuda.synchronize()
+            dt = time.perf_counter() - t
+            for s in slots:
+                eng.release(s)
+            return dt
+
+        def prefill():
+            ids = rand_ids(n_prefill)
+            best = None
+            for _ in range(3):
+                s = eng.acquire()
+                torch.cuda.synchronize()
+                t = time.perf_counter()
+                ops.argmax(eng.step([StepEntry(s, ids, [n_prefill - 1])]), next_tok[:1])
+                torch.cuda.synchronize()
+                dt = time.perf_counter() - t
+                eng.release(s)
+                best = dt if best is None else min(best, dt)
+            return best
+
+        if name == "duvulix":
+            step_bytes = lambda b: duvulix_step_bytes(raw, esize, b, args.context)[0]
+            params = duvulix_step_bytes(raw, esize, 0, 0)[1]
+        else:
+            step_bytes = lambda b: weight_bytes_per_step(cfg, esize) + b * args.context * kv_bytes_per_token(cfg, esize)
+            params = weight_bytes_per_step(cfg, esize) // esize
+        rec = {"decode": {}, "weights_gb": round(params * esize / 1e9, 3)}
+        for b in batches:
+            dt = decode(b, args.steps, args.warmup)
+            ms = dt / args.steps * 1e3
+            gbs = step_bytes(b) / (ms * 1e-3) / 1e9
+            rec["decode"][str(b)] = {"tokens_per_s": round(b * args.steps / dt, 1), "ms_per_step": round(ms, 4),
+                                     "gb_per_step": round(step_bytes(b) / 1e9, 3), "frac_of_hbm_peak": round(gbs / HBM_PEAK_GBS, 4),
+                                     "frac_of_read_kernel": round(gbs / read_gbs, 4)}
+            print(f"[bench] {name}: decode batch {b} context {args.context}: {ms:.3f} ms a step, {gbs:.0f} GB/s", file=sys.stderr, flush=True)
+        if not args.no_prefill:
+            dt = prefill()
+            flops = 2.0 * params * n_prefill
+            rec["prefill"] = {"tokens": n_prefill, "ms": round(dt * 1e3, 3), "tokens_per_s": round(n_prefill / dt, 1),
+                              "matrix_flops_frac_of_peak": round(flops / dt / PEAK_FLOPS["bf16" if esize == 2 else "fp32"], 4)}
+            print(f"[bench] {name}: prefill of {n_prefill} tokens: {dt * 1e3:.2f} ms", file=sys.stderr, flush=True)
+        if args.perf:
+            slots = filled(args.batch)
+            ids = rand_ids(args.batch)
+            rec["timers_decode"] = timer_table(eng, lambda: [eng.step([StepEntry(s, [ids[j]], [0]) for j, s in enumerate(slots)])
+                                                            for _ in range(8)], f"{name}, decode batch {args.batch}")
+            for s in slots:
+                eng.release(s)
+            pid = rand_ids(n_prefill)
+
+            def one_prompt():
+                for _ in range(3):
+                    s = eng.acquire()
+                    eng.step([StepEntry(s, pid, [n_prefill - 1])])
+                    eng.release(s)
+            rec["timers_prefill"] = timer_table(eng, one_prompt, f"{name}, prefill of {n_prefill}")
+        out[name] = rec
+        del eng
+        torch.cuda.empty_cache()
+    d = out["duvulix"]["decode"][str(args.batch)]
+    print(json.dumps({
+        "metric": f"Duvulix layer shapes (4 layers, width 4096): decode tok/s at batch {args.batch}, context {args.context}",
+        "value": d["tokens_per_s"], "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": d["ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16" if esize == 2 else "fp32", "data": "synthetic",
+        "config": {"model": "Duvulix layer shapes beside MiniCPM4-8B layer shapes, 4 layers each, random weights",
+                   "global_batch": args.batch, "seq_len": args.context, "parallelism": "1gpu",
+                   "hip_graph": bool(args.hip_graph), "duvulix": config_duvulix()},
+        "read_kernel_gbs": round(read_gbs, 1), "models": out}))
+
+
 def other_scenarios(args, dev):
-    """The two further workloads, each one JSON line of the same shape."""
+    """The further workloads, each one JSON line of the same shape."""
+    if args.scenario == "duvulix":
+        duvulix_scenario(args, dev)
+        return
     import torch
     from cpmcu_amd import Engine, EngineOptions, StepEntry
     from cpmcu_amd.config import MiniCPMConfig
