@@ -182,3 +182,266 @@ extern "C" const char* cpmcu_attention_general(const void* q, void* out, int dty
     CPMCU_LAUNCH_CHECK("attention_general");
     return nullptr;
 }
+
+// ===========================================================================
+// The same attention in bf16 on the matrix cores (v_mfma_f32_16x16x32_bf16), for prompts and single tokens.
+//
+// One wavefront owns one query token, one kv head and up to 16 of its query heads, and a share of the
+// token's visible keys (split over blockIdx.z for steps of few tokens, and over the 4 wavefronts of a workgroup
+// when NW = 4).  Keys are visited in chunks of 32, as they lie in their pages:
+//   S^T = K . Q^T     A = 16 keys x 32 features straight from the page, B = Q^T read from LDS (written there
+//                     once per token: a head of several hundred features does not fit registers beside the
+//                     output), looped over the key size at run time
+//   P^T = exp2(S^T c - m) in float per head, running maximum and sum
+//   O^T += V^T . P^T  A = V^T, 16 features x 32 keys a tile; the output of up to DTM tiles stays in registers
+// The mask is causal, and with chunk > 0 the keys before the start of the query's chunk are skipped (whole
+// 32-key chunks) or masked.  Output: out (bf16) when n_splits == 1, else unnormalised shares part_o
+// [token][head][split][hdv] and part_ml [token][head][split] = (max, sum) for the merge kernel below.
+// ===========================================================================
+typedef __bf16 gbf16x8_t __attribute__((ext_vector_type(8)));
+typedef float gfloatx4_t __attribute__((ext_vector_type(4)));
+
+template <int DTM, int NW, int TW>
+__global__ __launch_bounds__(NW * TW * 64) void attention_general_mfma_kernel(
+    const bf16_t* __restrict__ q, bf16_t* __restrict__ out, float* __restrict__ part_o, float2* __restrict__ part_ml,
+    const bf16_t* __restrict__ kpool, const bf16_t* __restrict__ vtpool, PagedView pv,
+    const int* __restrict__ positions, const int* __restrict__ tok_slot, int nh, int nkv, int hdk, int hdv,
+    int pool_hdk, int pool_hdv, float scale_log2e, int chunk, int n_splits, int n_tokens) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    static_assert(NW == 1 || TW == 1, "either the wavefronts of a workgroup share a token or each has its own");
+    const int ksteps = (pool_hdk + 31) >> 5, dtn = pool_hdv >> 4;
+    const int kvh = blockIdx.y % nkv, ht = blockIdx.y / nkv, split = blockIdx.z;
+    const int wave_id = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    const int wave = TW > 1 ? 0 : wave_id;
+    int t = blockIdx.x * TW + (TW > 1 ? wave_id : 0);
+    const bool live = t < n_tokens;
+    if (!live) t = n_tokens - 1;
+    const int lane = threadIdx.x & 63, n = lane & 15, g = lane >> 4;
+    const int G = nh / nkv;
+    const int head = kvh * G + ht * 16 + n;
+    const bool head_ok = ht * 16 + n < G;
+    const int pos = positions[t], slot = tok_slot[t];
+
+    // Q^T fragments of this wavefront's token: [ksteps][lane] of 8 features
+    gbf16x8_t* qs = (gbf16x8_t*)smem + (long)(TW > 1 ? wave_id : 0) * ksteps * 64;
+    for (int ks = wave; ks < ksteps; ks += NW) {
+        gbf16x8_t v = {0, 0, 0, 0, 0, 0, 0, 0};
+        const int d = ks * 32 + g * 8;
+        if (head_ok && d < hdk) v = *(const gbf16x8_t*)(q + ((long)t * nh + head) * hdk + d);
+        qs[ks * 64 + lane] = v;
+    }
+    __syncthreads();
+
+    const int first_key = chunk > 0 ? pos - pos % chunk : 0;
+    const int cfirst = first_key >> 5;
+    const int total_chunks = (pos >> 5) + 1 - cfirst;
+    const int per_split = (total_chunks + n_splits - 1) / n_splits;
+    const int c0 = split * per_split, c1 = min(c0 + per_split, total_chunks);
+
+    gfloatx4_t acc[DTM];
+#pragma unroll
+    for (int dt = 0; dt < DTM; ++dt) acc[dt] = gfloatx4_t{0.f, 0.f, 0.f, 0.f};
+    float m = -INFINITY, l = 0.f;
+    const int lane_off = (g * 16 + n) * 8;
+    const long kchunk = 32L * pool_hdk, vchunk = 32L * pool_hdv;
+    const int tile1 = (pool_hdk >> 3) * 128;                      // the second tile of 16 key slots
+
+    for (int c = c0 + wave; c < c1; c += NW) {
+        const int key0 = (cfirst + c) << 5;
+        const long pchunk = paged_row(pv, slot, key0) >> 5;
+        const bf16_t* kp = kpool + (pchunk * nkv + kvh) * kchunk + lane_off;
+        const bf16_t* vp = vtpool + (pchunk * nkv + kvh) * vchunk + lane_off;
+        gfloatx4_t st0 = {0.f, 0.f, 0.f, 0.f}, st1 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll 2
+        for (int ks = 0; ks < ksteps; ++ks) {
+            gbf16x8_t k0 = {0, 0, 0, 0, 0, 0, 0, 0}, k1 = {0, 0, 0, 0, 0, 0, 0, 0};
+            if (ks * 32 + g * 8 < pool_hdk) {
+                k0 = *(const gbf16x8_t*)(kp + ks * 512);
+                k1 = *(const gbf16x8_t*)(kp + tile1 + ks * 512);
+            }
+            const gbf16x8_t qv = qs[ks * 64 + lane];
+            st0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(k0, qv, st0, 0, 0, 0);
+            st1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(k1, qv, st1, 0, 0, 0);
+        }
+        // lane (head n, g): st0[e] is key key0 + 8g + e, st1[e] is key key0 + 8g + 4 + e
+        if (key0 + 31 > pos || key0 < first_key) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const int ka = key0 + 8 * g + e, kb = ka + 4;
+                if (ka > pos || ka < first_key) st0[e] = -INFINITY;
+                if (kb > pos || kb < first_key) st1[e] = -INFINITY;
+            }
+        }
+        float mx = fmaxf(fmaxf(fmaxf(st0[0], st0[1]), fmaxf(st0[2], st0[3])),
+                         fmaxf(fmaxf(st1[0], st1[1]), fmaxf(st1[2], st1[3])));
+        mx = rows_max(mx);
+        const float m_new = fmaxf(m, mx * scale_log2e);
+        const float m_ref = m_new == -INFINITY ? 0.f : m_new;
+        const float corr = exp2f(m - m_ref);
+        float rs = 0.f;
+        gbf16x8_t pb;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const float p0 = exp2f(__builtin_fmaf(st0[e], scale_log2e, -m_ref));
+            const float p1 = exp2f(__builtin_fmaf(st1[e], scale_log2e, -m_ref));
+            rs += p0 + p1;
+            pb[e] = (__bf16)p0;
+            pb[4 + e] = (__bf16)p1;
+        }
+        rs = rows_sum(rs);
+        l = l * corr + rs;
+        m = m_new;
+#pragma unroll
+        for (int dt = 0; dt < DTM; ++dt) {
+            if (dt < dtn) {
+                const gbf16x8_t vf = *(const gbf16x8_t*)(vp + dt * 512);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) acc[dt][e] *= corr;
+                acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pb, acc[dt], 0, 0, 0);
+            }
+        }
+    }
+
+    if (NW > 1) {
+        // merge the wavefronts' running results through LDS (behind the Q fragments)
+        float* ml_s = (float*)(smem + (long)ksteps * 64 * 16);
+        float* acc_s = ml_s + NW * 16 * 2;
+        __syncthreads();
+        if (g == 0) {
+            ml_s[(wave * 16 + n) * 2] = m;
+            ml_s[(wave * 16 + n) * 2 + 1] = l;
+        }
+#pragma unroll
+        for (int dt = 0; dt < DTM; ++dt)
+#pragma unroll
+            for (int i = 0; i < 4; ++i) acc_s[((wave * DTM + dt) * 4 + i) * 64 + lane] = acc[dt][i];
+        __syncthreads();
+        float m_all = -INFINITY;
+#pragma unroll
+        for (int w = 0; w < NW; ++w)
+            if (ml_s[(w * 16 + n) * 2 + 1] > 0.f) m_all = fmaxf(m_all, ml_s[(w * 16 + n) * 2]);
+        float l_all = 0.f;
+        float sw[NW];
+#pragma unroll
+        for (int w = 0; w < NW; ++w) {
+            sw[w] = ml_s[(w * 16 + n) * 2 + 1] > 0.f ? exp2f(ml_s[(w * 16 + n) * 2] - m_all) : 0.f;
+            l_all += sw[w] * ml_s[(w * 16 + n) * 2 + 1];
+        }
+        m = m_all;
+        l = l_all;
+#pragma unroll
+        for (int dt = 0; dt < DTM; ++dt) {
+            if (dt % NW != wave) continue;
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                float a = 0.f;
+#pragma unroll
+                for (int w = 0; w < NW; ++w) a += sw[w] * acc_s[((w * DTM + dt) * 4 + i) * 64 + lane];
+                acc[dt][i] = a;
+            }
+        }
+    }
+    if (!head_ok || !live) return;
+    // lane (head n, g): acc[dt][i] is O[head][dt*16 + 4g + i]
+    if (n_splits == 1) {
+        const float inv = 1.0f / l;
+        bf16_t* o = out + ((long)t * nh + head) * hdv;
+#pragma unroll
+        for (int dt = 0; dt < DTM; ++dt) {
+            if (dt >= dtn || (NW > 1 && dt % NW != wave)) continue;
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                if (dt * 16 + 4 * g + i < hdv) o[dt * 16 + 4 * g + i] = f32_to_bf16(acc[dt][i] * inv);
+        }
+    } else {
+        const long idx = ((long)t * nh + head) * n_splits + split;
+        float* o = part_o + idx * hdv;
+#pragma unroll
+        for (int dt = 0; dt < DTM; ++dt) {
+            if (dt >= dtn || (NW > 1 && dt % NW != wave)) continue;
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                if (dt * 16 + 4 * g + i < hdv) o[dt * 16 + 4 * g + i] = acc[dt][i];
+        }
+        if (g == 0 && wave == 0) part_ml[idx] = make_float2(m, l);
+    }
+}
+
+// out[token][head][:] = sum_s 2^(m_s - m) o_s / sum_s 2^(m_s - m) l_s over up to 64 shares (a share without keys
+// has l = 0): lane s holds share s's (max, sum), the common maximum and the denominator are wave reductions.
+__global__ void attention_general_merge_kernel(const float* __restrict__ part_o, const float2* __restrict__ part_ml,
+                                               bf16_t* __restrict__ out, int hdv, int n_splits) {
+    const long row = blockIdx.x;
+    const float2* ml = part_ml + row * n_splits;
+    const float* po = part_o + row * n_splits * hdv;
+    const int lane = threadIdx.x & 63;
+    float2 v = make_float2(-INFINITY, 0.f);
+    if (lane < n_splits) v = ml[lane];
+    const bool has = v.y > 0.f;
+    const float m = wave_max(has ? v.x : -INFINITY);
+    const float wv = has ? exp2f(v.x - m) : 0.f;
+    const float inv = 1.0f / wave_sum(wv * v.y);
+    for (int d = threadIdx.x; d < hdv; d += blockDim.x) {
+        float a = 0.f;
+        for (int s = 0; s < n_splits; ++s)
+            a += __int_as_float(__builtin_amdgcn_readlane(__float_as_int(wv), s)) * po[(long)s * hdv + d];
+        out[row * hdv + d] = f32_to_bf16(a * inv);
+    }
+}
+
+extern "C" const char* cpmcu_attention_general_mfma(const void* q, void* out, float* part_o, float* part_ml, int n,
+                                                    int nh, int nkv, int hdk, int hdv, int pool_hdk, int pool_hdv,
+                                                    float scale, int chunk, const void* kpool, const void* vtpool,
+                                                    const int* page_table, int table_width, int page_size,
+                                                    const int* positions, const int* tok_slot, int n_splits,
+                                                    hipStream_t stream) {
+    CPMCU_REQUIRE(n > 0 && nh > 0 && nkv > 0 && nh % nkv == 0, "attention_general_mfma: bad shape n=%d heads=%d kv_heads=%d", n, nh, nkv);
+    CPMCU_REQUIRE(hdk > 0 && hdk % 8 == 0 && hdk <= 1024 && hdv > 0 && hdv <= 512,
+                  "attention_general_mfma: key size %d (a multiple of 8 up to 1024) / value size %d (up to 512) have no "
+                  "matrix-core kernel; the plain kernel takes the rest", hdk, hdv);
+    CPMCU_REQUIRE(pool_hdk >= hdk && pool_hdv >= hdv && pool_hdk % 16 == 0 && pool_hdv % 16 == 0 && page_size % 32 == 0,
+                  "attention_general_mfma: the cache holds heads in steps of 16 features and pages of a multiple of 32 tokens");
+    CPMCU_REQUIRE(n_splits >= 1 && n_splits <= 64 && (n_splits == 1 || (part_o && part_ml)),
+                  "attention_general_mfma: %d shares of the keys (1..64 are taken)", n_splits);
+    CPMCU_REQUIRE(chunk >= 0, "attention_general_mfma: mask chunk %d", chunk);
+    const int G = nh / nkv, HT = (G + 15) / 16;
+    CPMCU_REQUIRE((long)nkv * HT <= 65535, "attention_general_mfma: too many head tiles");
+    PagedView pv{page_table, table_width, page_size};
+    const float sl = scale * 1.4426950408889634f;
+    const int ksteps = (pool_hdk + 31) / 32, dtn = pool_hdv / 16;
+    const int dtm = dtn <= 4 ? 4 : dtn <= 8 ? 8 : dtn <= 16 ? 16 : 32;
+    const long q_bytes = (long)ksteps * 64 * 16;
+    // few tokens: 4 wavefronts share a token's keys (while their merge fits LDS); many: a wavefront a token, 4
+    // neighbours a workgroup (while their Q fragments fit LDS)
+    const int nw = (n <= 256 && dtm <= 8) ? 4 : 1;
+    const int tw = (nw == 1 && n_splits == 1 && n >= 64 && 4 * q_bytes <= 48 * 1024) ? 4 : 1;
+    const long lds = (tw > 1 ? tw * q_bytes : q_bytes) + (nw > 1 ? (nw * 16 * 2 + (long)nw * dtm * 4 * 64) * 4 : 0);
+    CPMCU_REQUIRE(lds <= 64 * 1024, "attention_general_mfma: %ld bytes of LDS", lds);
+    dim3 grid((n + tw - 1) / tw, nkv * HT, n_splits);
+#define LAUNCH(DTMv, NWv, TWv)                                                                                   \
+    attention_general_mfma_kernel<DTMv, NWv, TWv><<<grid, NWv * TWv * 64, lds, stream>>>(                        \
+        (const bf16_t*)q, (bf16_t*)out, part_o, (float2*)part_ml, (const bf16_t*)kpool, (const bf16_t*)vtpool, pv, \
+        positions, tok_slot, nh, nkv, hdk, hdv, pool_hdk, pool_hdv, sl, chunk, n_splits, n)
+#define BY_SHAPE(DTMv)                         \
+    do {                                       \
+        if (tw == 4) LAUNCH(DTMv, 1, 4);       \
+        else LAUNCH(DTMv, 1, 1);               \
+    } while (0)
+    if (nw == 4) {
+        if (dtm == 4) LAUNCH(4, 4, 1);
+        else LAUNCH(8, 4, 1);
+    } else if (dtm == 4) BY_SHAPE(4);
+    else if (dtm == 8) BY_SHAPE(8);
+    else if (dtm == 16) BY_SHAPE(16);
+    else BY_SHAPE(32);
+#undef BY_SHAPE
+#undef LAUNCH
+    CPMCU_LAUNCH_CHECK("attention_general_mfma");
+    if (n_splits > 1) {
+        const unsigned rows = (unsigned)((long)n * nh);
+        attention_general_merge_kernel<<<rows, hdv > 128 ? 256 : (hdv > 64 ? 128 : 64), 0, stream>>>(
+            part_o, (const float2*)part_ml, (bf16_t*)out, hdv, n_splits);
+        CPMCU_LAUNCH_CHECK("attention_general_merge");
+    }
+    return nullptr;
+}

@@ -972,11 +972,74 @@ def attention(q, out, nh, nkv, hd, scale, kpool, vpool, page_table, page_size, c
                     sel_blocks, sel_count, block_size)
 
 
+def attention_general_mfma_ok(q: torch.Tensor, hdk: int, hdv: int, page_size: int) -> bool:
+    return q.dtype == torch.bfloat16 and hdk % 8 == 0 and hdk <= 1024 and hdv <= 512 and page_size % 32 == 0
+
+
+def attention_general_splits(n_tokens: int, nkv: int, group: int, pool_hdv: int, max_keys: int) -> int:
+    """Shares of a token's keys for attention_general_mfma in steps of few tokens: as attention_splits says, and
+    four times as many where a workgroup is one wavefront (values too wide for its four to merge through LDS)."""
+    s = attention_splits(n_tokens, nkv, group, max_keys)
+    if pool_hdv > 128 and n_tokens <= compute_units():
+        s = max(1, min(s * 4, 64, max_keys // 64))
+    return s
+
+
+def attention_general_mfma(q: torch.Tensor, out: torch.Tensor, nh: int, nkv: int, hdk: int, hdv: int, scale: float,
+                           kpool: torch.Tensor, vpool: torch.Tensor, page_table: torch.Tensor, page_size: int,
+                           positions: torch.Tensor, tok_slot: torch.Tensor, chunk: int = 0, n_splits: int = 1,
+                           part_o: Optional[torch.Tensor] = None, part_ml: Optional[torch.Tensor] = None):
+    """attention_general in bf16 on the matrix cores (key size a multiple of 8 up to 1024, value size up to 512).
+    With n_splits > 1 every token's visible keys are shared among n_splits workgroups and merged afterwards;
+    part_o float32 [n, nh, n_splits, hdv] and part_ml float32 [n, nh, n_splits, 2] are its scratch."""
+    _need(q, "attention q", torch.bfloat16, (None, nh * hdk))
+    n = q.shape[0]
+    _need(out, "attention out", torch.bfloat16, (n, nh * hdv))
+    _need(kpool, "attention key pool", torch.bfloat16, (None, page_size, None))
+    _need(vpool, "attention value pool", torch.bfloat16, (kpool.shape[0], page_size, None))
+    if kpool.shape[2] % nkv or vpool.shape[2] % nkv:
+        raise KernelError(f"attention_general: pools of {kpool.shape[2]} / {vpool.shape[2]} features do not hold {nkv} heads")
+    _need(page_table, "attention page table", torch.int32, (None, None))
+    _need(positions, "attention positions", torch.int32, (n,))
+    _need(tok_slot, "attention token slots", torch.int32, (n,))
+    if n_splits > 1:
+        _need(part_o, "attention partial outputs", torch.float32, (n, nh, n_splits, hdv))
+        _need(part_ml, "attention partial max/sum", torch.float32, (n, nh, n_splits, 2))
+    _check(_fn("attention_general", "cpmcu_attention_general_mfma")(
+        _p(q), _p(out), _p(part_o), _p(part_ml), c_int(n), c_int(nh), c_int(nkv), c_int(hdk), c_int(hdv),
+        c_int(kpool.shape[2] // nkv), c_int(vpool.shape[2] // nkv), c_float(scale), c_int(chunk), _p(kpool), _p(vpool),
+        _p(page_table), c_int(page_table.shape[1]), c_int(page_size), _p(positions), _p(tok_slot), c_int(n_splits),
+        _stream()))
+
+
+def reserve_attention_general(ws, dtype, nh: int, nkv: int, hdv: int, pool_hdv: int, max_keys: int, max_step_tokens: int):
+    """Ask the workspace for the shares of attention_any's split steps at their largest (they grow with the
+    context), so that no later step has to."""
+    if dtype != torch.bfloat16:
+        return
+    most = max((n * attention_general_splits(n, nkv, nh // nkv, pool_hdv, max_keys)
+                for n in range(1, min(max_step_tokens, compute_units()) + 1)), default=0)
+    if most > 1:
+        ws.get("attn.gpart_o", (most, nh, hdv), torch.float32)
+        ws.get("attn.gpart_ml", (most, nh, 2), torch.float32)
+
+
 def attention_any(q, out, nh, nkv, hdk, hdv, scale, kpool, vpool, page_table, page_size, ctx, chunk: int = 0):
     """Attention with key and value sizes of their own and an optional chunked mask, with the kernel that suits
     the step; writes ``out`` [n, nh*hdv]."""
-    if hdk == hdv and chunk == 0 and kpool.shape[2] == nkv * hdk:
+    if hdk == hdv and chunk == 0 and hdk <= 256 and kpool.shape[2] == nkv * hdk:
         attention(q, out, nh, nkv, hdk, scale, kpool, vpool, page_table, page_size, ctx)
+        return
+    if attention_general_mfma_ok(q, hdk, hdv, page_size):
+        n = q.shape[0]
+        keys = ctx.max_pos + 1 if chunk == 0 else min(ctx.max_pos + 1, chunk)
+        splits = attention_general_splits(n, nkv, nh // nkv, vpool.shape[2] // nkv, keys) if ctx.single_token else 1
+        part_o = part_ml = None
+        if splits > 1:
+            part_o = ctx.ws.get("attn.gpart_o", (n, nh, splits, hdv), torch.float32)
+            part_ml = ctx.ws.get("attn.gpart_ml", (n, nh, splits, 2), torch.float32)
+        attention_general_mfma(q, out, nh, nkv, hdk, hdv, scale, kpool, vpool, page_table, page_size, ctx.positions,
+                               ctx.tok_slot, chunk, splits, part_o, part_ml)
         return
     attention_general(q, out, nh, nkv, hdk, hdv, scale, kpool, vpool, page_table, page_size, ctx.positions,
                       ctx.tok_slot, chunk)

@@ -255,6 +255,10 @@ class GeneralAttention(Mixer):
                                    ("v", StreamSpec(self.nkv * _pad16(self.dv)))),
                           window=self.chunk or None)
 
+    def reserve_workspace(self, ws, rt: Runtime, max_step_tokens: int, max_slots: int):
+        keys = min(rt.max_seq_len, self.chunk) if self.chunk else rt.max_seq_len
+        ops.reserve_attention_general(ws, rt.dtype, self.nh, self.nkv, self.dv, _pad16(self.dv), keys, max_step_tokens)
+
     def forward(self, h, ctx: StepContext, cache: CacheView, writes_cache: bool = True):
         n, nh, nkv, dk, dv = h.shape[0], self.nh, self.nkv, self.dk, self.dv
         rot = self.position.rotary_params() if self.position is not None else None

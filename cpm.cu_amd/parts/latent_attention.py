@@ -78,6 +78,9 @@ class LatentAttention(Mixer):
     def cache_needs(self) -> CacheNeeds:
         return CacheNeeds(streams=(("k", StreamSpec(_pad16(self.dk))), ("v", StreamSpec(_pad16(self.rank)))))
 
+    def reserve_workspace(self, ws, rt: Runtime, max_step_tokens: int, max_slots: int):
+        ops.reserve_attention_general(ws, rt.dtype, self.nh, 1, self.rank, _pad16(self.rank), rt.max_seq_len, max_step_tokens)
+
     def _rotation(self):
         rot = self.position.rotary_params() if self.position is not None else None
         if self.rot and rot is None:

@@ -215,6 +215,35 @@ def test_attention_with_sizes_of_its_own_and_chunks(dtype, shape):
     close(out, want.reshape(T, H * dv), dtype)
 
 
+@pytest.mark.parametrize("splits", [1, 3, 16])
+@pytest.mark.parametrize("shape", [(4, 2, 48, 32, 40, 32, 150), (6, 1, 24, 40, 33, 64, 150), (2, 2, 80, 64, 0, 32, 150),
+                                   (20, 1, 136, 72, 64, 64, 150), (3, 1, 576, 512, 0, 64, 700), (35, 1, 320, 272, 100, 32, 90)])
+def test_matrix_core_attention_against_the_plain_kernel_and_the_plain_implementation(shape, splits):
+    """The bf16 kernel on the matrix cores: prompts (every token of a sequence at once, more than 64 tokens and
+    fewer) and shares of the keys that are merged; head groups larger than a tile of 16, sizes that are padded
+    in the cache, values wider than a wavefront's four can merge."""
+    from cpmcu_amd import ops
+    H, G, dk, dv, chunk, page, T = shape
+    torch.manual_seed(16)
+    q = torch.randn(T, H, dk).to(torch.bfloat16)
+    k = torch.randn(T, G, dk).to(torch.bfloat16)
+    v = torch.randn(T, G, dv).to(torch.bfloat16)
+    pages = [7, 2, 9, 0, 4, 11, 1, 3, 12, 5, 6, 8][:-(-T // page)]
+    kp, vp, table = _fill_cache(k, v, page, torch.bfloat16, pages)
+    pos, slot = dev(torch.arange(T, dtype=torch.int32)), dev(torch.ones(T, dtype=torch.int32))
+    s = torch.einsum("ihd,jhd->hij", q.double(), k.double().repeat_interleave(H // G, 1)) * dk ** -0.5
+    want = plain.softmax_attend(s, plain.visible(T, chunk or None), v.double().repeat_interleave(H // G, 1)).reshape(T, H * dv)
+    qd = dev(q.reshape(T, H * dk))
+    for rows in ((0, T), (T - 5, T), (T // 2, T // 2 + 1)):           # a prompt, a few tokens, a single token
+        a, b = rows
+        out = torch.empty(b - a, H * dv, dtype=torch.bfloat16, device=DEV)
+        po = torch.empty(b - a, H, splits, dv, device=DEV) if splits > 1 else None
+        pm = torch.empty(b - a, H, splits, 2, device=DEV) if splits > 1 else None
+        ops.attention_general_mfma(qd[a:b], out, H, G, dk, dv, dk ** -0.5, kp, vp, table, page, pos[a:b], slot[a:b], chunk,
+                                   splits, po, pm)
+        close(out, want[a:b], "bfloat16")
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_one_key_that_stands_out_at_the_edges_of_a_chunk(dtype):
     """The key at one position is made to dominate every query.  A query sees it exactly when it lies in the
@@ -234,6 +263,11 @@ def test_one_key_that_stands_out_at_the_edges_of_a_chunk(dtype):
         out = torch.empty(T, H * dv, dtype=DT[dtype], device=DEV)
         ops.attention_general(dev(q.reshape(T, H * dk), DT[dtype]), out, H, G, dk, dv, 1.0, kp, vp, table, page,
                               dev(torch.arange(T, dtype=torch.int32)), dev(torch.ones(T, dtype=torch.int32)), chunk)
+        if dtype == "bfloat16":       # the matrix-core kernel must see and not see exactly the same keys
+            out2 = torch.empty_like(out)
+            ops.attention_general_mfma(dev(q.reshape(T, H * dk), DT[dtype]), out2, H, G, dk, dv, 1.0, kp, vp, table, page,
+                                       dev(torch.arange(T, dtype=torch.int32)), dev(torch.ones(T, dtype=torch.int32)), chunk)
+            assert float((out2.float() - out.float()).abs().max()) < 0.05, (chunk, star)
         out = out.float().cpu().view(T, H, dv)
         vs = v[star, 0].to(DT[dtype]).float()
         sees = [p for p in range(T) if p >= star and (chunk == 0 or p // chunk == star // chunk)]
