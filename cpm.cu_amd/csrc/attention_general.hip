@@ -445,3 +445,158 @@ extern "C" const char* cpmcu_attention_general_mfma(const void* q, void* out, fl
     }
     return nullptr;
 }
+
+// ===========================================================================
+// Fused forms of the steps between a mixer's input projection and its attention.
+// ===========================================================================
+template <typename IT, typename OT>
+__device__ inline void rotate_run(const IT* __restrict__ s, OT* __restrict__ d, int width, int rot_dims, int pos,
+                                  const float* __restrict__ inv_freq, float mag, int mode, int f0, int lane, int nl) {
+    auto at = [&](int i) -> long {
+        if (mode == DST_ROWS) return i;
+        return mode == DST_KEYS ? key_d_offset(f0 + i) : value_d_offset(f0 + i);
+    };
+    const int half = rot_dims / 2;
+    for (int i = lane; i < half; i += nl) {
+        const float ang = (float)pos * inv_freq[i];
+        const float cs = cosf(ang) * mag, sn = sinf(ang) * mag;
+        const float u = to_f32(s[i]), v = to_f32(s[i + half]);
+        d[at(i)] = from_f32<OT>(u * cs - v * sn);
+        d[at(i + half)] = from_f32<OT>(v * cs + u * sn);
+    }
+    for (int i = rot_dims + lane; i < width; i += nl) d[at(i)] = from_f32<OT>(to_f32(s[i]));
+}
+
+// q, k, v of a stacked projection [q: nh*dk | k: nkv*dk | v: nkv*dv] in one launch: q rotated to plain rows,
+// k rotated into the key pages, v into the value pages.  grid (tokens, nh + 2 nkv) (nh alone without the cache).
+template <typename T>
+__global__ __launch_bounds__(64) void qkv_rotate_store_kernel(const T* __restrict__ qkv, long ld, T* __restrict__ q_out,
+                                                              int nh, int nkv, int dk, int dv, int rot_dims,
+                                                              const int* __restrict__ positions,
+                                                              const int* __restrict__ tok_slot,
+                                                              const float* __restrict__ inv_freq, float mag,
+                                                              T* __restrict__ kpool, T* __restrict__ vpool, PagedView pv,
+                                                              int pool_hdk, int pool_hdv) {
+    const long t = blockIdx.x;
+    const int y = blockIdx.y, lane = threadIdx.x;
+    const int pos = positions[t];
+    const T* row = qkv + t * ld;
+    if (y < nh) {
+        rotate_run(row + (long)y * dk, q_out + (t * nh + y) * dk, dk, rot_dims, pos, inv_freq, mag, DST_ROWS, 0, lane, 64);
+        return;
+    }
+    const long prow = paged_row(pv, tok_slot[t], pos);
+    if (y < nh + nkv) {
+        const int h = y - nh;
+        rotate_run(row + (long)(nh + h) * dk, kpool + key_index(prow, h, nkv, pool_hdk), dk, rot_dims, pos, inv_freq, mag,
+                   DST_KEYS, 0, lane, 64);
+    } else {
+        const int h = y - nh - nkv;
+        rotate_run(row + (long)(nh + nkv) * dk + (long)h * dv, vpool + value_index(prow, h, nkv, pool_hdv), dv, 0, pos,
+                   inv_freq, mag, DST_VALUES, 0, lane, 64);
+    }
+}
+
+extern "C" const char* cpmcu_qkv_rotate_store(const void* qkv, long ld, int dtype, void* q_out, int n, int nh, int nkv,
+                                              int dk, int dv, int rot_dims, const int* positions, const int* tok_slot,
+                                              const float* inv_freq, float mag, void* kpool, void* vpool,
+                                              const int* page_table, int table_width, int page_size, int pool_hdk,
+                                              int pool_hdv, int write_kv, hipStream_t stream) {
+    CPMCU_REQUIRE(n > 0 && nh > 0 && nkv > 0 && dk > 0 && dv > 0, "qkv_rotate_store: empty shape");
+    CPMCU_REQUIRE(rot_dims >= 0 && rot_dims % 2 == 0 && rot_dims <= dk && (rot_dims == 0 || inv_freq),
+                  "qkv_rotate_store: %d rotated features of %d", rot_dims, dk);
+    CPMCU_REQUIRE(ld >= (long)nh * dk + (write_kv ? (long)nkv * (dk + dv) : 0), "qkv_rotate_store: rows of %ld too short", ld);
+    CPMCU_REQUIRE(!write_kv || (kpool && vpool && page_table && page_size % 32 == 0 && pool_hdk % 16 == 0 &&
+                                pool_hdv % 16 == 0 && pool_hdk >= dk && pool_hdv >= dv),
+                  "qkv_rotate_store: the cache takes pages of a multiple of 32 tokens and head sizes in steps of 16");
+    const int heads = nh + (write_kv ? 2 * nkv : 0);
+    CPMCU_REQUIRE(heads <= 65535, "qkv_rotate_store: %d heads exceed the launch grid", heads);
+    PagedView pv{page_table, table_width, page_size};
+    dim3 grid(n, heads);
+    if (dtype == CPMCU_F32)
+        qkv_rotate_store_kernel<float><<<grid, 64, 0, stream>>>((const float*)qkv, ld, (float*)q_out, nh, nkv, dk, dv, rot_dims,
+                                                                positions, tok_slot, inv_freq, mag, (float*)kpool,
+                                                                (float*)vpool, pv, pool_hdk, pool_hdv);
+    else if (dtype == CPMCU_BF16)
+        qkv_rotate_store_kernel<bf16_t><<<grid, 64, 0, stream>>>((const bf16_t*)qkv, ld, (bf16_t*)q_out, nh, nkv, dk, dv,
+                                                                 rot_dims, positions, tok_slot, inv_freq, mag,
+                                                                 (bf16_t*)kpool, (bf16_t*)vpool, pv, pool_hdk, pool_hdv);
+    else
+        CPMCU_FAIL("qkv_rotate_store: unknown dtype %d", dtype);
+    CPMCU_LAUNCH_CHECK("qkv_rotate_store");
+    return nullptr;
+}
+
+// Latent attention: from a row [q heads: nh * (dim + rot) | down: rank + rot | ...] in one launch
+//   * y < nh: head y's rotated query part goes, rotated, behind the `rank` latent features of its query row
+//     q_out[t, y, rank:rank + rot] (the latent features themselves come from a product over heads);
+//   * y == nh (layers that own the cache): the latent c = rmsnorm(down[:rank]) * norm_w in float, into the key
+//     pages (features 0..rank) and the value pages, and the shared key part down[rank:], rotated, into the key
+//     pages behind it.
+template <typename T>
+__global__ __launch_bounds__(256) void latent_store_kernel(const T* __restrict__ proj, long ld, T* __restrict__ q_out,
+                                                           int nh, int dim, int rot, int rank,
+                                                           const float* __restrict__ norm_w, float eps,
+                                                           const int* __restrict__ positions,
+                                                           const int* __restrict__ tok_slot,
+                                                           const float* __restrict__ inv_freq, float mag,
+                                                           T* __restrict__ kpool, T* __restrict__ vpool, PagedView pv,
+                                                           int pool_hdk, int pool_hdv) {
+    __shared__ float red[17];
+    const long t = blockIdx.x;
+    const int y = blockIdx.y;
+    const int pos = positions[t];
+    const int qw = dim + rot, dk = rank + rot;
+    if (y < nh) {
+        rotate_run(proj + t * ld + (long)y * qw + dim, q_out + (t * nh + y) * dk + rank, rot, rot, pos, inv_freq, mag,
+                   DST_ROWS, 0, (int)threadIdx.x, (int)blockDim.x);
+        return;
+    }
+    const T* down = proj + t * ld + (long)nh * qw;
+    float ss = 0.f;
+    for (int c = threadIdx.x; c < rank; c += blockDim.x) {
+        const float v = to_f32(down[c]);
+        ss += v * v;
+    }
+    ss = block_sum(ss, red);
+    const float rs = 1.0f / sqrtf(ss / (float)rank + eps);
+    const long prow = paged_row(pv, tok_slot[t], pos);
+    T* kd = kpool + key_index(prow, 0, 1, pool_hdk);
+    T* vd = vpool + value_index(prow, 0, 1, pool_hdv);
+    for (int c = threadIdx.x; c < rank; c += blockDim.x) {
+        const T v = from_f32<T>(to_f32(down[c]) * rs * norm_w[c]);
+        kd[key_d_offset(c)] = v;
+        vd[value_d_offset(c)] = v;
+    }
+    rotate_run(down + rank, kd, rot, rot, pos, inv_freq, mag, DST_KEYS, rank, (int)threadIdx.x, (int)blockDim.x);
+}
+
+extern "C" const char* cpmcu_latent_store(const void* proj, long ld, int dtype, void* q_out, int n, int nh, int dim,
+                                          int rot, int rank, const float* norm_w, float eps, const int* positions,
+                                          const int* tok_slot, const float* inv_freq, float mag, void* kpool,
+                                          void* vpool, const int* page_table, int table_width, int page_size,
+                                          int pool_hdk, int pool_hdv, int write_cache, hipStream_t stream) {
+    CPMCU_REQUIRE(n > 0 && nh > 0 && dim > 0 && rank > 0 && rot >= 0 && rot % 2 == 0, "latent_store: bad shape");
+    CPMCU_REQUIRE(rot == 0 || inv_freq, "latent_store: frequencies missing");
+    CPMCU_REQUIRE(ld >= (long)nh * (dim + rot) + (write_cache ? rank + rot : 0), "latent_store: rows of %ld too short", ld);
+    CPMCU_REQUIRE(!write_cache || (norm_w && kpool && vpool && page_table && page_size % 32 == 0 && pool_hdk % 16 == 0 &&
+                                   pool_hdv % 16 == 0 && pool_hdk >= rank + rot && pool_hdv >= rank),
+                  "latent_store: the cache takes pages of a multiple of 32 tokens and head sizes in steps of 16");
+    CPMCU_REQUIRE(nh < 65535, "latent_store: %d heads exceed the launch grid", nh);
+    if (!write_cache && rot == 0) return nullptr;
+    PagedView pv{page_table, table_width, page_size};
+    dim3 grid(n, nh + (write_cache ? 1 : 0));
+    const int block = rank >= 256 ? 256 : 64;
+    if (dtype == CPMCU_F32)
+        latent_store_kernel<float><<<grid, block, 0, stream>>>((const float*)proj, ld, (float*)q_out, nh, dim, rot, rank,
+                                                               norm_w, eps, positions, tok_slot, inv_freq, mag,
+                                                               (float*)kpool, (float*)vpool, pv, pool_hdk, pool_hdv);
+    else if (dtype == CPMCU_BF16)
+        latent_store_kernel<bf16_t><<<grid, block, 0, stream>>>((const bf16_t*)proj, ld, (bf16_t*)q_out, nh, dim, rot, rank,
+                                                                norm_w, eps, positions, tok_slot, inv_freq, mag,
+                                                                (bf16_t*)kpool, (bf16_t*)vpool, pv, pool_hdk, pool_hdv);
+    else
+        CPMCU_FAIL("latent_store: unknown dtype %d", dtype);
+    CPMCU_LAUNCH_CHECK("latent_store");
+    return nullptr;
+}

@@ -154,6 +154,91 @@ extern "C" const char* cpmcu_gemm_nt_heads(const void* X, long ldx, long hsx, co
     return nullptr;
 }
 
+// The product head by head in bf16 on the matrix cores (v_mfma_f32_16x16x32_bf16).  A workgroup of 4
+// wavefronts owns, for one head, 64 rows x 64 columns (WM = 4: a wavefront a tile of 16 rows) or 16 rows x 256
+// columns (WM = 1, steps of few rows: a wavefront 64 columns); a wavefront holds 4 tiles of 16 x 16 results.
+// Operands come straight from memory, 16 bytes a lane: lane (r, g) of a tile reads row r, columns k0 + 8g .. + 8,
+// of X and of W alike (W [N, K] row-major is the transposed operand as it lies).  K is a multiple of 8 and
+// rows start on 16-byte borders (the launcher checks).
+typedef __bf16 hbf16x8_t __attribute__((ext_vector_type(8)));
+typedef float hfloatx4_t __attribute__((ext_vector_type(4)));
+
+template <int WM>
+__global__ __launch_bounds__(256) void gemm_heads_mfma_kernel(const bf16_t* __restrict__ X, long ldx, long hsx,
+                                                              const bf16_t* __restrict__ W, bf16_t* __restrict__ Y,
+                                                              long ldy, long hsy, const bf16_t* __restrict__ gate,
+                                                              long ldg, int M, int N, int K) {
+    const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    const int lane = threadIdx.x & 63, r = lane & 15, g = lane >> 4;
+    const int h = blockIdx.z;
+    const int m0 = blockIdx.y * (WM == 4 ? 64 : 16) + (WM == 4 ? wave * 16 : 0);
+    const int n0 = blockIdx.x * (WM == 4 ? 64 : 256) + (WM == 4 ? 0 : wave * 64);
+    if (m0 >= M || n0 >= N) return;
+    const bf16_t* xp = X + (long)h * hsx + (long)min(m0 + r, M - 1) * ldx + g * 8;
+    const bf16_t* wp = W + (long)h * N * K + g * 8;
+    const bool row_ok = m0 + r < M;
+    hfloatx4_t acc[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) acc[j] = hfloatx4_t{0.f, 0.f, 0.f, 0.f};
+    long wrow[4];
+    bool col_ok[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        col_ok[j] = n0 + 16 * j + r < N;
+        wrow[j] = (long)min(n0 + 16 * j + r, N - 1) * K;
+    }
+#pragma unroll 2
+    for (int k0 = 0; k0 < K; k0 += 32) {
+        const bool k_ok = k0 + g * 8 < K;
+        hbf16x8_t a = {0, 0, 0, 0, 0, 0, 0, 0};
+        if (k_ok && row_ok) a = *(const hbf16x8_t*)(xp + k0);
+        hbf16x8_t b[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            b[j] = hbf16x8_t{0, 0, 0, 0, 0, 0, 0, 0};
+            if (k_ok && col_ok[j]) b[j] = *(const hbf16x8_t*)(wp + wrow[j] + k0);
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b[j], acc[j], 0, 0, 0);
+    }
+    // lane (column r, g): acc[j][i] is the result of row m0 + 4g + i, column n0 + 16j + r
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int m = m0 + 4 * g + i;
+        if (m >= M) continue;
+        float gs = 1.f;
+        if (gate) gs = 1.0f / (1.0f + expf(-to_f32(gate[(long)m * ldg + h])));
+        bf16_t* yr = Y + (long)h * hsy + (long)m * ldy;
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+            if (n0 + 16 * j + r < N) yr[n0 + 16 * j + r] = f32_to_bf16(gs * acc[j][i]);
+    }
+}
+
+extern "C" const char* cpmcu_gemm_nt_heads_mfma(const void* X, long ldx, long hsx, const void* W, void* Y, long ldy,
+                                                long hsy, const void* gate, long ldg, int M, int H, int N, int K,
+                                                hipStream_t stream) {
+    CPMCU_REQUIRE(M > 0 && H > 0 && N > 0 && K > 0, "gemm_heads_mfma: empty shape M=%d heads=%d N=%d K=%d", M, H, N, K);
+    CPMCU_REQUIRE(K % 8 == 0 && ldx % 8 == 0 && hsx % 8 == 0 && ((uintptr_t)X % 16 == 0) && ((uintptr_t)W % 16 == 0),
+                  "gemm_heads_mfma: K, the row stride and the head stride of X must be multiples of 8 elements and "
+                  "the operands start on 16-byte borders (K=%d, %ld, %ld)", K, ldx, hsx);
+    CPMCU_REQUIRE(ldx >= (H - 1) * hsx + K && ldy >= (H - 1) * hsy + N && (!gate || ldg >= H),
+                  "gemm_heads_mfma: rows of %ld / %ld elements cannot hold %d heads", ldx, ldy, H);
+    CPMCU_REQUIRE(H <= 65535, "gemm_heads_mfma: %d heads exceed the launch grid", H);
+    if (M <= 16) {
+        dim3 grid((N + 255) / 256, 1, H);
+        gemm_heads_mfma_kernel<1><<<grid, 256, 0, stream>>>((const bf16_t*)X, ldx, hsx, (const bf16_t*)W, (bf16_t*)Y, ldy,
+                                                            hsy, (const bf16_t*)gate, ldg, M, N, K);
+    } else {
+        dim3 grid((N + 63) / 64, (M + 63) / 64, H);
+        CPMCU_REQUIRE(grid.y <= 65535, "gemm_heads_mfma: M=%d too large for one launch", M);
+        gemm_heads_mfma_kernel<4><<<grid, 256, 0, stream>>>((const bf16_t*)X, ldx, hsx, (const bf16_t*)W, (bf16_t*)Y, ldy,
+                                                            hsy, (const bf16_t*)gate, ldg, M, N, K);
+    }
+    CPMCU_LAUNCH_CHECK("gemm_nt_heads_mfma");
+    return nullptr;
+}
+
 // ===========================================================================
 // Skinny product for decode steps (bf16, at most 64 rows of X):
 //   Y[m,N] = alpha * X[m,K] . W[N,K]^T

@@ -110,6 +110,60 @@ __global__ __launch_bounds__(256) void branch_norm_add_norm_kernel(float* __rest
     }
 }
 
+// The same with the row held in registers (H <= 1024 * VPT): one trip to memory for the branch's slices and the
+// residual, all loads of a thread in flight together (a loop of dependent passes over the row costs a step of
+// few rows ten times as much).
+template <typename BT, typename OT, int VPT>
+__global__ __launch_bounds__(1024) void branch_norm_add_norm_reg_kernel(float* __restrict__ x, const BT* __restrict__ b,
+                                                                        int nparts, long part_stride,
+                                                                        const float* __restrict__ wb, float eps_b,
+                                                                        const float* __restrict__ w, float eps,
+                                                                        OT* __restrict__ out,
+                                                                        const int* __restrict__ rows, int H) {
+    __shared__ float red[17];
+    const long r = rows ? rows[blockIdx.x] : blockIdx.x;
+    float* xr = x + r * H;
+    const BT* br = b + r * H;
+    float bv[VPT], xv[VPT], wbv[VPT], wv[VPT];
+#pragma unroll
+    for (int i = 0; i < VPT; ++i) {
+        const int c = threadIdx.x + i * 1024;
+        bv[i] = 0.f;
+        xv[i] = c < H ? xr[c] : 0.f;
+        wbv[i] = c < H ? wb[c] : 0.f;
+        wv[i] = (c < H && out) ? w[c] : 0.f;
+    }
+    for (int p = 0; p < nparts; ++p) {
+#pragma unroll
+        for (int i = 0; i < VPT; ++i) {
+            const int c = threadIdx.x + i * 1024;
+            if (c < H) bv[i] += to_f32(br[(long)p * part_stride + c]);
+        }
+    }
+    float sb = 0.f;
+#pragma unroll
+    for (int i = 0; i < VPT; ++i) sb += bv[i] * bv[i];
+    sb = block_sum(sb, red);
+    const float rb = 1.0f / sqrtf(sb / (float)H + eps_b);
+    float sx = 0.f;
+#pragma unroll
+    for (int i = 0; i < VPT; ++i) {
+        const int c = threadIdx.x + i * 1024;
+        xv[i] += bv[i] * rb * wbv[i];
+        if (!rows && c < H) xr[c] = xv[i];
+        sx += xv[i] * xv[i];
+    }
+    if (!out) return;
+    sx = block_sum(sx, red);
+    const float rx = 1.0f / sqrtf(sx / (float)H + eps);
+    OT* orow = out + (long)blockIdx.x * H;
+#pragma unroll
+    for (int i = 0; i < VPT; ++i) {
+        const int c = threadIdx.x + i * 1024;
+        if (c < H) orow[c] = from_f32<OT>(xv[i] * rx * wv[i]);
+    }
+}
+
 extern "C" const char* cpmcu_branch_norm_add_norm(float* x, const void* b, int b_dtype, int nparts, long part_stride,
                                                   const float* wb, float eps_b, const float* w, float eps, void* out,
                                                   int out_dtype, const int* rows, int n_out, int H,
@@ -118,8 +172,17 @@ extern "C" const char* cpmcu_branch_norm_add_norm(float* x, const void* b, int b
     CPMCU_REQUIRE(x && b && wb && (!out || w), "branch_norm_add_norm: a pointer is missing");
     CPMCU_REQUIRE(!rows || out, "branch_norm_add_norm: a list of rows needs an output");
 #define LAUNCH(BT, OT)                                                                                              \
-    branch_norm_add_norm_kernel<BT, OT><<<n_out, 256, 0, stream>>>(x, (const BT*)b, nparts, part_stride, wb, eps_b, \
-                                                                   w, eps, (OT*)out, rows, H)
+    do {                                                                                                            \
+        if (H <= 2048)                                                                                              \
+            branch_norm_add_norm_reg_kernel<BT, OT, 2><<<n_out, 1024, 0, stream>>>(                                 \
+                x, (const BT*)b, nparts, part_stride, wb, eps_b, w, eps, (OT*)out, rows, H);                        \
+        else if (H <= 8192)                                                                                         \
+            branch_norm_add_norm_reg_kernel<BT, OT, 8><<<n_out, 1024, 0, stream>>>(                                 \
+                x, (const BT*)b, nparts, part_stride, wb, eps_b, w, eps, (OT*)out, rows, H);                        \
+        else                                                                                                        \
+            branch_norm_add_norm_kernel<BT, OT><<<n_out, 256, 0, stream>>>(x, (const BT*)b, nparts, part_stride, wb, \
+                                                                           eps_b, w, eps, (OT*)out, rows, H);       \
+    } while (0)
     if (b_dtype == CPMCU_F32 && out_dtype == CPMCU_F32) LAUNCH(float, float);
     else if (b_dtype == CPMCU_F32 && out_dtype == CPMCU_BF16) LAUNCH(float, bf16_t);
     else if (b_dtype == CPMCU_BF16 && out_dtype == CPMCU_BF16) LAUNCH(bf16_t, bf16_t);
@@ -160,11 +223,61 @@ __global__ __launch_bounds__(256) void poly_norm_kernel(const ZT* __restrict__ z
     }
 }
 
+// The same with the row held in registers (F <= 1024 * VPT).
+template <typename ZT, typename OT, int VPT>
+__global__ __launch_bounds__(1024) void poly_norm_reg_kernel(const ZT* __restrict__ z, int nparts, long part_stride,
+                                                             const float* __restrict__ coef, OT* __restrict__ out,
+                                                             int F, float eps) {
+    __shared__ float red[17];
+    const long r = blockIdx.x;
+    const ZT* zr = z + r * F;
+    float zv[VPT];
+#pragma unroll
+    for (int i = 0; i < VPT; ++i) zv[i] = 0.f;
+    for (int p = 0; p < nparts; ++p) {
+#pragma unroll
+        for (int i = 0; i < VPT; ++i) {
+            const int c = threadIdx.x + i * 1024;
+            if (c < F) zv[i] += to_f32(zr[(long)p * part_stride + c]);
+        }
+    }
+    float s2 = 0.f, s4 = 0.f, s6 = 0.f;
+#pragma unroll
+    for (int i = 0; i < VPT; ++i) {
+        const float v2 = zv[i] * zv[i];
+        s2 += v2;
+        s4 += v2 * v2;
+        s6 += v2 * v2 * v2;
+    }
+    s2 = block_sum(s2, red);
+    s4 = block_sum(s4, red);
+    s6 = block_sum(s6, red);
+    const float inv = 1.0f / (float)F;
+    const float a = coef[0] / sqrtf(s2 * inv + eps), b = coef[1] / sqrtf(s4 * inv + eps),
+                cc = coef[2] / sqrtf(s6 * inv + eps), e = coef[3];
+    OT* orow = out + r * F;
+#pragma unroll
+    for (int i = 0; i < VPT; ++i) {
+        const int c = threadIdx.x + i * 1024;
+        if (c < F) orow[c] = from_f32<OT>(((cc * zv[i] + b) * zv[i] + a) * zv[i] + e);
+    }
+}
+
 extern "C" const char* cpmcu_poly_norm(const void* z, int z_dtype, int nparts, long part_stride, const float* coef,
                                        void* out, int out_dtype, int n, int F, float eps, hipStream_t stream) {
     CPMCU_REQUIRE(n > 0 && F > 0 && nparts >= 1, "poly_norm: empty shape rows=%d width=%d", n, F);
-#define LAUNCH(ZT, OT) \
-    poly_norm_kernel<ZT, OT><<<n, 256, 0, stream>>>((const ZT*)z, nparts, part_stride, coef, (OT*)out, F, eps)
+#define LAUNCH(ZT, OT)                                                                                          \
+    do {                                                                                                        \
+        if (F <= 4096)                                                                                          \
+            poly_norm_reg_kernel<ZT, OT, 4><<<n, 1024, 0, stream>>>((const ZT*)z, nparts, part_stride, coef,    \
+                                                                    (OT*)out, F, eps);                          \
+        else if (F <= 16384)                                                                                    \
+            poly_norm_reg_kernel<ZT, OT, 16><<<n, 1024, 0, stream>>>((const ZT*)z, nparts, part_stride, coef,   \
+                                                                     (OT*)out, F, eps);                         \
+        else                                                                                                    \
+            poly_norm_kernel<ZT, OT><<<n, 256, 0, stream>>>((const ZT*)z, nparts, part_stride, coef, (OT*)out,  \
+                                                            F, eps);                                            \
+    } while (0)
     if (z_dtype == CPMCU_F32 && out_dtype == CPMCU_F32) LAUNCH(float, float);
     else if (z_dtype == CPMCU_F32 && out_dtype == CPMCU_BF16) LAUNCH(float, bf16_t);
     else if (z_dtype == CPMCU_BF16 && out_dtype == CPMCU_BF16) LAUNCH(bf16_t, bf16_t);

@@ -613,6 +613,70 @@ def rotate_copy(src: torch.Tensor, src_off: int, src_head_stride: int, heads: in
         _p(page_table), c_int(tw), c_int(page_size), c_int(pool_heads), c_int(pool_hd), _stream()))
 
 
+def qkv_rotate_store(qkv: torch.Tensor, q_out: torch.Tensor, nh: int, nkv: int, dk: int, dv: int, rot_dims: int,
+                     positions: torch.Tensor, tok_slot: torch.Tensor, inv_freq: Optional[torch.Tensor], mag: float,
+                     kpool: Optional[torch.Tensor], vpool: Optional[torch.Tensor], page_table: Optional[torch.Tensor],
+                     page_size: int, write_kv: bool = True):
+    """rotate_copy three times in one launch: a row of qkv is [q: nh*dk | k: nkv*dk | v: nkv*dv]; q goes, rotated
+    in its first rot_dims features, to q_out [n, nh*dk], k rotated into the key pages, v into the value pages
+    (pools whose heads may be padded to a multiple of 16 features)."""
+    ld = _ld(qkv, "qkv")
+    n = qkv.shape[0]
+    if qkv.shape[1] < nh * dk + (nkv * (dk + dv) if write_kv else 0):
+        raise KernelError(f"qkv_rotate_store: rows of {qkv.shape[1]} cannot hold {nh} query heads and {nkv} key/value heads")
+    _need(q_out, "qkv q_out", qkv.dtype, (n, nh * dk))
+    _need(positions, "qkv positions", torch.int32, (n,))
+    if rot_dims:
+        _need(inv_freq, "qkv inv_freq", torch.float32, (rot_dims // 2,))
+    tw = pk = pv = 0
+    if write_kv:
+        _need(tok_slot, "qkv token slots", torch.int32, (n,))
+        _need(page_table, "qkv page table", torch.int32, (None, None))
+        _need(kpool, "qkv key pool", qkv.dtype, (None, page_size, None))
+        _need(vpool, "qkv value pool", qkv.dtype, (kpool.shape[0], page_size, None))
+        if kpool.shape[2] % nkv or vpool.shape[2] % nkv:
+            raise KernelError(f"qkv_rotate_store: pools of {kpool.shape[2]} / {vpool.shape[2]} features do not hold {nkv} heads")
+        tw, pk, pv = page_table.shape[1], kpool.shape[2] // nkv, vpool.shape[2] // nkv
+    _check(_fn("attention_general", "cpmcu_qkv_rotate_store")(
+        _p(qkv), c_long(ld), c_int(_code(qkv)), _p(q_out), c_int(n), c_int(nh), c_int(nkv), c_int(dk), c_int(dv),
+        c_int(rot_dims), _p(positions), _p(tok_slot), _p(inv_freq), c_float(mag), _p(kpool if write_kv else None),
+        _p(vpool if write_kv else None), _p(page_table if write_kv else None), c_int(tw), c_int(page_size), c_int(pk),
+        c_int(pv), c_int(1 if write_kv else 0), _stream()))
+
+
+def latent_store(proj: torch.Tensor, q_out: torch.Tensor, nh: int, dim: int, rot: int, rank: int,
+                 norm_w: Optional[torch.Tensor], eps: float, positions: torch.Tensor, tok_slot: torch.Tensor,
+                 inv_freq: Optional[torch.Tensor], mag: float, kpool: Optional[torch.Tensor],
+                 vpool: Optional[torch.Tensor], page_table: Optional[torch.Tensor], page_size: int,
+                 write_cache: bool = True):
+    """Latent attention's steps between projection and attention in one launch.  A row of proj is
+    [nh heads of (dim plain | rot rotated) | rank + rot of the down projection (if write_cache) | ...]:
+    every head's rotated part goes, rotated, to q_out[t, head, rank:rank+rot] (q_out [n, nh*(rank+rot)]); with
+    write_cache the latent rmsnorm(down[:rank]) * norm_w goes into the key pages (features 0..rank) and the value
+    pages, and down[rank:], rotated, into the key pages behind it."""
+    ld = _ld(proj, "latent projection")
+    n = proj.shape[0]
+    if proj.shape[1] < nh * (dim + rot) + (rank + rot if write_cache else 0):
+        raise KernelError(f"latent_store: rows of {proj.shape[1]} are too short")
+    _need(q_out, "latent q_out", proj.dtype, (n, nh * (rank + rot)))
+    _need(positions, "latent positions", torch.int32, (n,))
+    if rot:
+        _need(inv_freq, "latent inv_freq", torch.float32, (rot // 2,))
+    tw = pk = pv = 0
+    if write_cache:
+        _need(norm_w, "latent norm weight", torch.float32, (rank,))
+        _need(tok_slot, "latent token slots", torch.int32, (n,))
+        _need(page_table, "latent page table", torch.int32, (None, None))
+        _need(kpool, "latent key pool", proj.dtype, (None, page_size, None))
+        _need(vpool, "latent value pool", proj.dtype, (kpool.shape[0], page_size, None))
+        tw, pk, pv = page_table.shape[1], kpool.shape[2], vpool.shape[2]
+    _check(_fn("attention_general", "cpmcu_latent_store")(
+        _p(proj), c_long(ld), c_int(_code(proj)), _p(q_out), c_int(n), c_int(nh), c_int(dim), c_int(rot), c_int(rank),
+        _p(norm_w if write_cache else None), c_float(eps), _p(positions), _p(tok_slot), _p(inv_freq), c_float(mag),
+        _p(kpool if write_cache else None), _p(vpool if write_cache else None), _p(page_table if write_cache else None),
+        c_int(tw), c_int(page_size), c_int(pk), c_int(pv), c_int(1 if write_cache else 0), _stream()))
+
+
 def attention_general(q: torch.Tensor, out: torch.Tensor, nh: int, nkv: int, hdk: int, hdv: int, scale: float,
                       kpool: torch.Tensor, vpool: torch.Tensor, page_table: torch.Tensor, page_size: int,
                       positions: torch.Tensor, tok_slot: torch.Tensor, chunk: int = 0):
@@ -637,9 +701,10 @@ def attention_general(q: torch.Tensor, out: torch.Tensor, nh: int, nkv: int, hdk
 
 
 def gemm_heads(x: torch.Tensor, x_off: int, x_head_stride: int, w: torch.Tensor, out: torch.Tensor, out_off: int,
-               out_head_stride: int, gate: Optional[torch.Tensor] = None):
+               out_head_stride: int, gate: Optional[torch.Tensor] = None, plain: bool = False):
     """out[m, out_off + h*out_head_stride + :N] = x[m, x_off + h*x_head_stride + :K] . w[h]^T for every head h;
-    w [H, N, K].  With ``gate`` [m, H] head h's rows are multiplied by sigmoid(gate[m, h])."""
+    w [H, N, K].  With ``gate`` [m, H] head h's rows are multiplied by sigmoid(gate[m, h]).  bf16 runs on the
+    matrix cores when K and the strides of x are multiples of 8 (``plain``: the scalar kernel all the same)."""
     ldx, ldy = _ld(x, "heads x"), _ld(out, "heads out")
     M = x.shape[0]
     _need(w, "heads weight", x.dtype, (None, None, None))
@@ -655,6 +720,12 @@ def gemm_heads(x: torch.Tensor, x_off: int, x_head_stride: int, w: torch.Tensor,
             raise KernelError(f"heads gate: {gate.dtype} {tuple(gate.shape)}, expected {x.dtype} {(M, H)}")
     xp = c_void_p(x.data_ptr() + x_off * x.element_size())
     op = c_void_p(out.data_ptr() + out_off * out.element_size())
+    if (x.dtype == torch.bfloat16 and out.dtype == torch.bfloat16 and not plain and K % 8 == 0 and ldx % 8 == 0
+            and x_head_stride % 8 == 0 and xp.value % 16 == 0 and w.data_ptr() % 16 == 0):
+        _check(_fn("gemm", "cpmcu_gemm_nt_heads_mfma")(xp, c_long(ldx), c_long(x_head_stride), _p(w), op, c_long(ldy),
+                                                       c_long(out_head_stride), _p(gate), c_long(ldg), c_int(M),
+                                                       c_int(H), c_int(N), c_int(K), _stream()))
+        return
     _check(_fn("gemm", "cpmcu_gemm_nt_heads")(xp, c_long(ldx), c_long(x_head_stride), _p(w), op, c_long(ldy),
                                               c_long(out_head_stride), _p(gate), c_long(ldg), c_int(_code(x)),
                                               c_int(_code(out)), c_int(M), c_int(H), c_int(N), c_int(K), _stream()))

@@ -271,14 +271,9 @@ class GeneralAttention(Mixer):
         with ctx.timed("attn_qkv_rope"):
             qkv = self.qkv.forward(h, ctx, "attn.qkv", rows=None if writes_cache else nh * dk)
             q = ctx.ws.get("attn.q", (n, nh * dk), self.rt.dtype)
-            ops.rotate_copy(qkv, 0, dk, nh, dk, rd, ctx.positions, inv_freq, mag, q, ops.ROTATE_TO_ROWS, 0, dk)
-            if writes_cache:
-                kp, vp = cache.streams["k"], cache.streams["v"]
-                paged = dict(tok_slot=ctx.tok_slot, page_table=cache.page_table, page_size=cache.page_size, pool_heads=nkv)
-                ops.rotate_copy(qkv, nh * dk, dk, nkv, dk, rd, ctx.positions, inv_freq, mag, kp, ops.ROTATE_TO_KEYS,
-                                pool_hd=kp.shape[2] // nkv, **paged)
-                ops.rotate_copy(qkv, (nh + nkv) * dk, dv, nkv, dv, 0, ctx.positions, None, 1.0, vp,
-                                ops.ROTATE_TO_VALUES, pool_hd=vp.shape[2] // nkv, **paged)
+            ops.qkv_rotate_store(qkv, q, nh, nkv, dk, dv, rd, ctx.positions, ctx.tok_slot, inv_freq, mag,
+                                 cache.streams["k"], cache.streams["v"], cache.page_table, cache.page_size,
+                                 write_kv=writes_cache)
         out = ctx.ws.get("attn.out", (n, nh * dv), self.rt.dtype)
         with ctx.timed("attn_core"):
             ops.attention_any(q, out, nh, nkv, dk, dv, self.scale, cache.streams["k"], cache.streams["v"],

@@ -102,23 +102,11 @@ class LatentAttention(Mixer):
             # the query in the latent space: [W_uk[h]^T q_plain | rotated q_rot] per head
             q = ctx.ws.get("lat.q", (n, H * self.dk), self.rt.dtype)
             ops.gemm_heads(proj, 0, self.qw, self.uk_t, q, 0, self.dk)
-            if self.rot:
-                ops.rotate_copy(proj, self.dim, self.qw, H, self.rot, self.rot, ctx.positions, inv_freq, mag, q,
-                                ops.ROTATE_TO_ROWS, dst_off=R, dst_head_stride=self.dk)
-            off = H * self.qw
-            if writes_cache:
-                c = ctx.ws.get("lat.c", (n, R), self.rt.dtype)
-                ops.rms_norm_groups(proj[:, off:off + R], self.down_norm, self.eps, c)
-                paged = dict(tok_slot=ctx.tok_slot, page_table=cache.page_table, page_size=cache.page_size, pool_heads=1)
-                kp, vp = cache.streams["k"], cache.streams["v"]
-                ops.rotate_copy(c, 0, 0, 1, R, 0, ctx.positions, None, 1.0, kp, ops.ROTATE_TO_KEYS, dst_off=0,
-                                pool_hd=kp.shape[2], **paged)
-                if self.rot:
-                    ops.rotate_copy(proj, off + R, 0, 1, self.rot, self.rot, ctx.positions, inv_freq, mag, kp,
-                                    ops.ROTATE_TO_KEYS, dst_off=R, pool_hd=kp.shape[2], **paged)
-                ops.rotate_copy(c, 0, 0, 1, R, 0, ctx.positions, None, 1.0, vp, ops.ROTATE_TO_VALUES, dst_off=0,
-                                pool_hd=vp.shape[2], **paged)
-                off += R + self.rot
+            # rotated query parts, the normed latent and the rotated shared key part, to their places: one launch
+            ops.latent_store(proj, q, H, self.dim, self.rot, R, self.down_norm if writes_cache else None, self.eps,
+                             ctx.positions, ctx.tok_slot, inv_freq, mag, cache.streams["k"], cache.streams["v"],
+                             cache.page_table, cache.page_size, write_cache=writes_cache)
+            off = H * self.qw + ((R + self.rot) if writes_cache else 0)
         o_lat = ctx.ws.get("lat.o_lat", (n, H * R), self.rt.dtype)
         with ctx.timed("attn_core"):
             ops.attention_any(q, o_lat, H, 1, self.dk, R, self.scale, cache.streams["k"], cache.streams["v"],

@@ -311,3 +311,25 @@ def test_products_head_by_head_with_gate(dtype):
         want = xs @ w[h].double().T * torch.sigmoid(gate[:, 1 + h].double())[:, None]
         close(out[:, 16 + h * (N + 16):16 + h * (N + 16) + N], want, dtype)
     assert float(out[:, :16].abs().max()) == 0.0
+
+
+@pytest.mark.parametrize("shape", [(70, 3, 40, 24), (8, 5, 200, 64), (1, 2, 16, 512), (300, 2, 130, 136)])
+def test_products_head_by_head_on_the_matrix_cores(shape):
+    from cpmcu_amd import ops
+    torch.manual_seed(10)
+    M, H, N, K = shape
+    x = torch.randn(M, 8 + H * (K + 8)).to(torch.bfloat16)
+    w = (torch.randn(H, N, K) * 0.3).to(torch.bfloat16)
+    gate = torch.randn(M, H).to(torch.bfloat16)
+    for gt in (None, dev(gate)):
+        out = torch.zeros(M, H * (N + 3), dtype=torch.bfloat16, device=DEV)
+        twin = torch.zeros_like(out)
+        ops.gemm_heads(dev(x), 8, K + 8, dev(w), out, 0, N + 3, gate=gt)
+        ops.gemm_heads(dev(x), 8, K + 8, dev(w), twin, 0, N + 3, gate=gt, plain=True)
+        for h in range(H):
+            want = x[:, 8 + h * (K + 8):8 + h * (K + 8) + K].double() @ w[h].double().T
+            if gt is not None:
+                want = want * torch.sigmoid(gate[:, h].double())[:, None]
+            close(out[:, h * (N + 3):h * (N + 3) + N], want, "bfloat16")
+            assert float(out[:, h * (N + 3) + N:(h + 1) * (N + 3)].abs().max()) == 0.0
+        assert float((out.float() - twin.float()).abs().max()) <= 0.02 * float(twin.float().abs().max())
