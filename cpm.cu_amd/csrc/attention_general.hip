@@ -201,7 +201,11 @@ extern "C" const char* cpmcu_attention_general(const void* q, void* out, int dty
 typedef __bf16 gbf16x8_t __attribute__((ext_vector_type(8)));
 typedef float gfloatx4_t __attribute__((ext_vector_type(4)));
 
-template <int DTM, int NW, int TW>
+// VS (features split): the 4 wavefronts of a workgroup all visit all of the workgroup's keys; each computes the
+// scores' share of a quarter of the key features (the shares are summed through LDS) and owns a quarter of the
+// value features (DTM tiles of 16 from tile wave * DTM on): for keys and values too wide to keep a whole
+// output row in one wavefront's registers.  Every key and value is loaded once, and nothing is merged at the end.
+template <int DTM, int NW, int TW, bool VS>
 __global__ __launch_bounds__(NW * TW * 64) void attention_general_mfma_kernel(
     const bf16_t* __restrict__ q, bf16_t* __restrict__ out, float* __restrict__ part_o, float2* __restrict__ part_ml,
     const bf16_t* __restrict__ kpool, const bf16_t* __restrict__ vtpool, PagedView pv,
@@ -246,22 +250,58 @@ __global__ __launch_bounds__(NW * TW * 64) void attention_general_mfma_kernel(
     const long kchunk = 32L * pool_hdk, vchunk = 32L * pool_hdv;
     const int tile1 = (pool_hdk >> 3) * 128;                      // the second tile of 16 key slots
 
-    for (int c = c0 + wave; c < c1; c += NW) {
+    const int dt0 = VS ? wave * DTM : 0;
+    const int kq = VS ? (ksteps + NW - 1) / NW : ksteps;
+    const int ks_a = VS ? wave * kq : 0, ks_b = VS ? min(ks_a + kq, ksteps) : ksteps;
+    float* sc_s = (float*)(smem + (long)ksteps * 64 * 16);        // VS: partial scores, behind the Q fragments
+    int parity = 0;
+    for (int c = VS ? c0 : c0 + wave; c < c1; c += VS ? 1 : NW) {
         const int key0 = (cfirst + c) << 5;
         const long pchunk = paged_row(pv, slot, key0) >> 5;
         const bf16_t* kp = kpool + (pchunk * nkv + kvh) * kchunk + lane_off;
         const bf16_t* vp = vtpool + (pchunk * nkv + kvh) * vchunk + lane_off;
+        // the values are asked for first: they arrive behind the scores' work.  No load stands in a branch
+        // (lanes beyond the head's features read its first ones and are zeroed by a select), so that the
+        // compiler keeps several steps' loads in flight.
+        gbf16x8_t vf[DTM];
+#pragma unroll
+        for (int dt = 0; dt < DTM; ++dt) vf[dt] = *(const gbf16x8_t*)(vp + min(dt0 + dt, dtn - 1) * 512);
         gfloatx4_t st0 = {0.f, 0.f, 0.f, 0.f}, st1 = {0.f, 0.f, 0.f, 0.f};
-#pragma unroll 2
-        for (int ks = 0; ks < ksteps; ++ks) {
-            gbf16x8_t k0 = {0, 0, 0, 0, 0, 0, 0, 0}, k1 = {0, 0, 0, 0, 0, 0, 0, 0};
-            if (ks * 32 + g * 8 < pool_hdk) {
-                k0 = *(const gbf16x8_t*)(kp + ks * 512);
-                k1 = *(const gbf16x8_t*)(kp + tile1 + ks * 512);
-            }
+        const gbf16x8_t zero8 = {0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll 6
+        for (int ks = ks_a; ks < ks_b; ++ks) {
+            const bool ok = ks * 32 + g * 8 < pool_hdk;
+            const int off = ok ? ks * 512 : -g * 128;
+            gbf16x8_t k0 = *(const gbf16x8_t*)(kp + off);
+            gbf16x8_t k1 = *(const gbf16x8_t*)(kp + tile1 + off);
+            k0 = ok ? k0 : zero8;
+            k1 = ok ? k1 : zero8;
             const gbf16x8_t qv = qs[ks * 64 + lane];
             st0 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(k0, qv, st0, 0, 0, 0);
             st1 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(k1, qv, st1, 0, 0, 0);
+        }
+        if (VS) {
+            // every wavefront took a quarter of the key features: the four partial scores meet in LDS (two
+            // buffers in turn, so that one barrier a chunk is enough)
+            float* sc = sc_s + (parity ? NW * 8 * 64 : 0);
+            parity ^= 1;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                sc[(wave * 8 + e) * 64 + lane] = st0[e];
+                sc[(wave * 8 + 4 + e) * 64 + lane] = st1[e];
+            }
+            __syncthreads();
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                float a0 = 0.f, a1 = 0.f;
+#pragma unroll
+                for (int w = 0; w < NW; ++w) {
+                    a0 += sc[(w * 8 + e) * 64 + lane];
+                    a1 += sc[(w * 8 + 4 + e) * 64 + lane];
+                }
+                st0[e] = a0;
+                st1[e] = a1;
+            }
         }
         // lane (head n, g): st0[e] is key key0 + 8g + e, st1[e] is key key0 + 8g + 4 + e
         if (key0 + 31 > pos || key0 < first_key) {
@@ -293,16 +333,15 @@ __global__ __launch_bounds__(NW * TW * 64) void attention_general_mfma_kernel(
         m = m_new;
 #pragma unroll
         for (int dt = 0; dt < DTM; ++dt) {
-            if (dt < dtn) {
-                const gbf16x8_t vf = *(const gbf16x8_t*)(vp + dt * 512);
+            if (dt0 + dt < dtn) {
 #pragma unroll
                 for (int e = 0; e < 4; ++e) acc[dt][e] *= corr;
-                acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf, pb, acc[dt], 0, 0, 0);
+                acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[dt], pb, acc[dt], 0, 0, 0);
             }
         }
     }
 
-    if (NW > 1) {
+    if (NW > 1 && !VS) {
         // merge the wavefronts' running results through LDS (behind the Q fragments)
         float* ml_s = (float*)(smem + (long)ksteps * 64 * 16);
         float* acc_s = ml_s + NW * 16 * 2;
@@ -348,20 +387,20 @@ __global__ __launch_bounds__(NW * TW * 64) void attention_general_mfma_kernel(
         bf16_t* o = out + ((long)t * nh + head) * hdv;
 #pragma unroll
         for (int dt = 0; dt < DTM; ++dt) {
-            if (dt >= dtn || (NW > 1 && dt % NW != wave)) continue;
+            if (dt0 + dt >= dtn || (NW > 1 && !VS && dt % NW != wave)) continue;
 #pragma unroll
             for (int i = 0; i < 4; ++i)
-                if (dt * 16 + 4 * g + i < hdv) o[dt * 16 + 4 * g + i] = f32_to_bf16(acc[dt][i] * inv);
+                if ((dt0 + dt) * 16 + 4 * g + i < hdv) o[(dt0 + dt) * 16 + 4 * g + i] = f32_to_bf16(acc[dt][i] * inv);
         }
     } else {
         const long idx = ((long)t * nh + head) * n_splits + split;
         float* o = part_o + idx * hdv;
 #pragma unroll
         for (int dt = 0; dt < DTM; ++dt) {
-            if (dt >= dtn || (NW > 1 && dt % NW != wave)) continue;
+            if (dt0 + dt >= dtn || (NW > 1 && !VS && dt % NW != wave)) continue;
 #pragma unroll
             for (int i = 0; i < 4; ++i)
-                if (dt * 16 + 4 * g + i < hdv) o[dt * 16 + 4 * g + i] = acc[dt][i];
+                if ((dt0 + dt) * 16 + 4 * g + i < hdv) o[(dt0 + dt) * 16 + 4 * g + i] = acc[dt][i];
         }
         if (g == 0 && wave == 0) part_ml[idx] = make_float2(m, l);
     }
@@ -383,7 +422,16 @@ __global__ void attention_general_merge_kernel(const float* __restrict__ part_o,
     const float inv = 1.0f / wave_sum(wv * v.y);
     for (int d = threadIdx.x; d < hdv; d += blockDim.x) {
         float a = 0.f;
-        for (int s = 0; s < n_splits; ++s)
+        int s = 0;
+        for (; s + 8 <= n_splits; s += 8) {          // eight shares' loads in flight
+            float v8[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) v8[u] = po[(long)(s + u) * hdv + d];
+#pragma unroll
+            for (int u = 0; u < 8; ++u)
+                a += __int_as_float(__builtin_amdgcn_readlane(__float_as_int(wv), s + u)) * v8[u];
+        }
+        for (; s < n_splits; ++s)
             a += __int_as_float(__builtin_amdgcn_readlane(__float_as_int(wv), s)) * po[(long)s * hdv + d];
         out[row * hdv + d] = f32_to_bf16(a * inv);
     }
@@ -409,32 +457,37 @@ extern "C" const char* cpmcu_attention_general_mfma(const void* q, void* out, fl
     PagedView pv{page_table, table_width, page_size};
     const float sl = scale * 1.4426950408889634f;
     const int ksteps = (pool_hdk + 31) / 32, dtn = pool_hdv / 16;
-    const int dtm = dtn <= 4 ? 4 : dtn <= 8 ? 8 : dtn <= 16 ? 16 : 32;
     const long q_bytes = (long)ksteps * 64 * 16;
-    // few tokens: 4 wavefronts share a token's keys (while their merge fits LDS); many: a wavefront a token, 4
-    // neighbours a workgroup (while their Q fragments fit LDS)
-    const int nw = (n <= 256 && dtm <= 8) ? 4 : 1;
+    // values up to 128 features: few tokens: 4 wavefronts share a token's keys and merge through LDS; many: a
+    // wavefront a token, 4 neighbours a workgroup (while their Q fragments fit LDS).  Wider values: the 4
+    // wavefronts of a token's workgroup split the value features.
+    const bool vs = dtn > 8;
+    const int dtm = vs ? (dtn <= 16 ? 4 : 8) : (dtn <= 4 ? 4 : 8);
+    // (four wavefronts that merge through LDS need room there beside the Q fragments)
+    const long merge_bytes = (4 * 16 * 2 + 4L * dtm * 4 * 64) * 4;
+    const int nw = (vs || (n <= 256 && q_bytes + merge_bytes <= 64 * 1024)) ? 4 : 1;
     const int tw = (nw == 1 && n_splits == 1 && n >= 64 && 4 * q_bytes <= 48 * 1024) ? 4 : 1;
-    const long lds = (tw > 1 ? tw * q_bytes : q_bytes) + (nw > 1 ? (nw * 16 * 2 + (long)nw * dtm * 4 * 64) * 4 : 0);
+    const long lds = (tw > 1 ? tw * q_bytes : q_bytes) + ((nw > 1 && !vs) ? (nw * 16 * 2 + (long)nw * dtm * 4 * 64) * 4 : 0) +
+                     (vs ? 2L * nw * 8 * 64 * 4 : 0);
     CPMCU_REQUIRE(lds <= 64 * 1024, "attention_general_mfma: %ld bytes of LDS", lds);
     dim3 grid((n + tw - 1) / tw, nkv * HT, n_splits);
-#define LAUNCH(DTMv, NWv, TWv)                                                                                   \
-    attention_general_mfma_kernel<DTMv, NWv, TWv><<<grid, NWv * TWv * 64, lds, stream>>>(                        \
+#define LAUNCH(DTMv, NWv, TWv, VSv)                                                                              \
+    attention_general_mfma_kernel<DTMv, NWv, TWv, VSv><<<grid, NWv * TWv * 64, lds, stream>>>(                   \
         (const bf16_t*)q, (bf16_t*)out, part_o, (float2*)part_ml, (const bf16_t*)kpool, (const bf16_t*)vtpool, pv, \
         positions, tok_slot, nh, nkv, hdk, hdv, pool_hdk, pool_hdv, sl, chunk, n_splits, n)
-#define BY_SHAPE(DTMv)                         \
-    do {                                       \
-        if (tw == 4) LAUNCH(DTMv, 1, 4);       \
-        else LAUNCH(DTMv, 1, 1);               \
-    } while (0)
-    if (nw == 4) {
-        if (dtm == 4) LAUNCH(4, 4, 1);
-        else LAUNCH(8, 4, 1);
-    } else if (dtm == 4) BY_SHAPE(4);
-    else if (dtm == 8) BY_SHAPE(8);
-    else if (dtm == 16) BY_SHAPE(16);
-    else BY_SHAPE(32);
-#undef BY_SHAPE
+    if (vs) {
+        if (dtm == 4) LAUNCH(4, 4, 1, true);
+        else LAUNCH(8, 4, 1, true);
+    } else if (nw == 4) {
+        if (dtm == 4) LAUNCH(4, 4, 1, false);
+        else LAUNCH(8, 4, 1, false);
+    } else if (tw == 4) {
+        if (dtm == 4) LAUNCH(4, 1, 4, false);
+        else LAUNCH(8, 1, 4, false);
+    } else {
+        if (dtm == 4) LAUNCH(4, 1, 1, false);
+        else LAUNCH(8, 1, 1, false);
+    }
 #undef LAUNCH
     CPMCU_LAUNCH_CHECK("attention_general_mfma");
     if (n_splits > 1) {

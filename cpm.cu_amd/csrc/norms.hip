@@ -133,14 +133,31 @@ __global__ __launch_bounds__(1024) void branch_norm_add_norm_reg_kernel(float* _
         wbv[i] = c < H ? wb[c] : 0.f;
         wv[i] = (c < H && out) ? w[c] : 0.f;
     }
-    for (int p = 0; p < nparts; ++p) {
+    // four slices' loads are issued before any of them is added
+    int p = 0;
+    for (; p + 4 <= nparts; p += 4) {
+        float t4[4][VPT];
+#pragma unroll
+        for (int u = 0; u < 4; ++u)
+#pragma unroll
+            for (int i = 0; i < VPT; ++i) {
+                const int c = min((int)threadIdx.x + i * 1024, H - 1);  // clamped: no load in a branch
+                t4[u][i] = to_f32(br[(long)(p + u) * part_stride + c]);
+            }
+#pragma unroll
+        for (int i = 0; i < VPT; ++i) bv[i] += (t4[0][i] + t4[1][i]) + (t4[2][i] + t4[3][i]);
+    }
+    for (; p < nparts; ++p) {
 #pragma unroll
         for (int i = 0; i < VPT; ++i) {
-            const int c = threadIdx.x + i * 1024;
-            if (c < H) bv[i] += to_f32(br[(long)p * part_stride + c]);
+            const int c = min((int)threadIdx.x + i * 1024, H - 1);
+            bv[i] += to_f32(br[(long)p * part_stride + c]);
         }
     }
     float sb = 0.f;
+#pragma unroll
+    for (int i = 0; i < VPT; ++i)
+        if ((int)threadIdx.x + i * 1024 >= H) bv[i] = 0.f;
 #pragma unroll
     for (int i = 0; i < VPT; ++i) sb += bv[i] * bv[i];
     sb = block_sum(sb, red);
@@ -175,6 +192,9 @@ extern "C" const char* cpmcu_branch_norm_add_norm(float* x, const void* b, int b
     do {                                                                                                            \
         if (H <= 2048)                                                                                              \
             branch_norm_add_norm_reg_kernel<BT, OT, 2><<<n_out, 1024, 0, stream>>>(                                 \
+                x, (const BT*)b, nparts, part_stride, wb, eps_b, w, eps, (OT*)out, rows, H);                        \
+        else if (H <= 4096)                                                                                         \
+            branch_norm_add_norm_reg_kernel<BT, OT, 4><<<n_out, 1024, 0, stream>>>(                                 \
                 x, (const BT*)b, nparts, part_stride, wb, eps_b, w, eps, (OT*)out, rows, H);                        \
         else if (H <= 8192)                                                                                         \
             branch_norm_add_norm_reg_kernel<BT, OT, 8><<<n_out, 1024, 0, stream>>>(                                 \

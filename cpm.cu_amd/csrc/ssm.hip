@@ -12,12 +12,12 @@
 //
 // The scan walks a sequence's tokens in order; a workgroup owns one (sequence, head, 32 columns of P), a
 // column's N state values are spread over 8 neighbouring lanes, and the tokens' B, C, x and dt pass through
-// LDS in tiles of 16 tokens.
+// LDS in tiles of 16 or 32 tokens, the next tile asked for while the current one is worked on.
 #include "common.h"
 
 __device__ inline float silu_f(float z) { return z / (1.0f + expf(-z)); }
 
-// grid (sequences, token tiles of 64, channel blocks of 256 threads)
+// grid (sequences, token tiles of 16, channel blocks of 256 threads)
 template <typename UT>
 __global__ __launch_bounds__(256) void conv_silu_kernel(const UT* __restrict__ u, long ldu,
                                                         const float* __restrict__ weight,
@@ -30,7 +30,7 @@ __global__ __launch_bounds__(256) void conv_silu_kernel(const UT* __restrict__ u
     const int slot = seq_slot[b];
     const int c = blockIdx.z * blockDim.x + threadIdx.x;
     if (c >= C) return;
-    const int i0 = blockIdx.y * 64, i1 = min(i0 + 64, q);
+    const int i0 = blockIdx.y * 16, i1 = min(i0 + 16, q);
     const float* st = state + (long)slot * (taps - 1) * C + c;        // [slot][taps-1][C]
     const float bs = bias ? bias[c] : 0.f;
     for (int i = i0; i < i1; ++i) {
@@ -70,8 +70,9 @@ extern "C" const char* cpmcu_conv_silu(const void* u, long ldu, int u_dtype, con
                   n_seqs, max_q, C, taps);
     CPMCU_REQUIRE(ldu >= C, "conv_silu: rows of %ld elements cannot hold %d channels", ldu, C);
     CPMCU_REQUIRE(taps == 1 || state, "conv_silu: the state of the last inputs is missing");
-    const int cb = (C + 255) / 256, tb = (max_q + 63) / 64;
-    CPMCU_REQUIRE(tb <= 65535 && cb <= 65535, "conv_silu: shape exceeds the launch grid");
+    const int cb = (C + 255) / 256, tb = (max_q + 15) / 16;
+    CPMCU_REQUIRE(tb <= 65535 && cb <= 65535, "conv_silu: shape exceeds the launch grid (a step brings at most 1,048,560 "
+                  "tokens a sequence)");
     dim3 grid(n_seqs, tb, cb), grid2(n_seqs, cb);
     if (u_dtype == CPMCU_F32) {
         conv_silu_kernel<float><<<grid, 256, 0, stream>>>((const float*)u, ldu, weight, bias, state, out, cu_q, seq_slot, C, taps);
@@ -90,13 +91,14 @@ extern "C" const char* cpmcu_conv_silu(const void* u, long ldu, int u_dtype, con
 
 #define SCAN_PB 32       // columns of P a workgroup
 #define SCAN_L 8         // lanes a column: state index n = l + 8 i
-#define SCAN_TT 16       // tokens a tile in LDS
 
 __device__ inline float softplus_f(float v) { return fmaxf(v, 0.f) + log1pf(expf(-fabsf(v))); }
 
 // xbc: float [n, ldx] = [x: heads*P | B: groups*N | C: groups*N]; dt: raw step sizes [n, lddt] (first `heads`
 // columns at the given pointer); state: float [slots][heads][P][N]; y: float [n, heads*P].
-template <int NR, typename DT>
+// Tiles of TT tokens pass through LDS; while a tile is worked on, the next one's values are already asked for
+// (held in registers until the tile is done), so that the walk over a long prompt waits for memory once.
+template <int NR, int TT, typename DT>
 __global__ __launch_bounds__(256) void ssm_scan_kernel(const float* __restrict__ xbc, long ldx,
                                                        const DT* __restrict__ dt, long lddt,
                                                        const float* __restrict__ dt_bias,
@@ -104,10 +106,14 @@ __global__ __launch_bounds__(256) void ssm_scan_kernel(const float* __restrict__
                                                        float* __restrict__ state, float* __restrict__ y,
                                                        const int* __restrict__ cu_q, const int* __restrict__ seq_slot,
                                                        int heads, int P, int N, int groups, int write_state) {
-    __shared__ float Bs[SCAN_TT][NR * SCAN_L];
-    __shared__ float Cs[SCAN_TT][NR * SCAN_L];
-    __shared__ float xs[SCAN_TT][SCAN_PB];
-    __shared__ float dts[SCAN_TT], das[SCAN_TT];
+    constexpr int NS = NR * SCAN_L;                 // state values a column, padded
+    constexpr int BC = TT * NS / 256;               // B (and C) values a thread brings a tile
+    constexpr int XV = (TT * SCAN_PB + 255) / 256;  // x values a thread brings a tile
+    static_assert(TT * NS % 256 == 0 && TT <= 64, "tile shape");
+    __shared__ float Bs[TT][NS];
+    __shared__ float Cs[TT][NS];
+    __shared__ float xs[TT][SCAN_PB];
+    __shared__ float dts[TT], das[TT];
     const int b = blockIdx.x, h = blockIdx.y, p0 = blockIdx.z * SCAN_PB;
     const int start = cu_q[b], q = cu_q[b + 1] - start;
     const int slot = seq_slot[b];
@@ -124,25 +130,48 @@ __global__ __launch_bounds__(256) void ssm_scan_kernel(const float* __restrict__
         S[i] = (p_ok && n < N) ? sp[n] : 0.f;
     }
     const float A = expf(A_log[h]), bias = dt_bias[h], Dh = Dskip[h];
-    for (int t0 = 0; t0 < q; t0 += SCAN_TT) {
-        const int tn = min(SCAN_TT, q - t0);
-        __syncthreads();
-        for (int e = threadIdx.x; e < tn * NR * SCAN_L; e += 256) {
-            const int tt = e / (NR * SCAN_L), n = e % (NR * SCAN_L);
-            const float* row = xbc + (long)(start + t0 + tt) * ldx + inner + (long)g * N;
-            Bs[tt][n] = n < N ? row[n] : 0.f;
-            Cs[tt][n] = n < N ? row[(long)groups * N + n] : 0.f;
+    float rb[BC], rc[BC], rx[XV], rdt = 0.f;
+    auto fetch = [&](int t0) {
+        const int tn = min(TT, q - t0);
+#pragma unroll
+        for (int k = 0; k < BC; ++k) {
+            const int e = threadIdx.x + k * 256;
+            const int tt = e / NS, n = e % NS;
+            const bool ok = tt < tn && n < N;
+            const float* row = xbc + (long)(start + t0 + min(tt, tn - 1)) * ldx + inner + (long)g * N + min(n, N - 1);
+            rb[k] = ok ? row[0] : 0.f;
+            rc[k] = ok ? row[(long)groups * N] : 0.f;
         }
-        for (int e = threadIdx.x; e < tn * SCAN_PB; e += 256) {
+#pragma unroll
+        for (int k = 0; k < XV; ++k) {
+            const int e = threadIdx.x + k * 256;
             const int tt = e / SCAN_PB, pp = e % SCAN_PB;
-            xs[tt][pp] = p0 + pp < P ? xbc[(long)(start + t0 + tt) * ldx + (long)h * P + p0 + pp] : 0.f;
+            rx[k] = (tt < tn && p0 + pp < P) ? xbc[(long)(start + t0 + tt) * ldx + (long)h * P + p0 + pp] : 0.f;
+        }
+        if ((int)threadIdx.x < tn) rdt = to_f32(dt[(long)(start + t0 + threadIdx.x) * lddt + h]);
+    };
+    fetch(0);
+    for (int t0 = 0; t0 < q; t0 += TT) {
+        const int tn = min(TT, q - t0);
+        __syncthreads();
+#pragma unroll
+        for (int k = 0; k < BC; ++k) {
+            const int e = threadIdx.x + k * 256;
+            Bs[e / NS][e % NS] = rb[k];
+            Cs[e / NS][e % NS] = rc[k];
+        }
+#pragma unroll
+        for (int k = 0; k < XV; ++k) {
+            const int e = threadIdx.x + k * 256;
+            if (e < TT * SCAN_PB) xs[e / SCAN_PB][e % SCAN_PB] = rx[k];
         }
         if ((int)threadIdx.x < tn) {
-            const float d = softplus_f(to_f32(dt[(long)(start + t0 + threadIdx.x) * lddt + h]) + bias);
+            const float d = softplus_f(rdt + bias);
             dts[threadIdx.x] = d;
             das[threadIdx.x] = expf(-A * d);
         }
         __syncthreads();
+        if (t0 + TT < q) fetch(t0 + TT);
         for (int tt = 0; tt < tn; ++tt) {
             const float d = dts[tt], da = das[tt], xv = xs[tt][pl];
             const float dx = d * xv;
@@ -181,16 +210,16 @@ extern "C" const char* cpmcu_ssm_scan(const float* xbc, long ldx, const void* dt
     CPMCU_REQUIRE(heads <= 65535 && pb <= 65535, "ssm_scan: shape exceeds the launch grid");
     dim3 grid(n_seqs, heads, pb);
     const int need = (N + SCAN_L - 1) / SCAN_L;
-#define LAUNCH(NRv, DTv)                                                                                          \
-    ssm_scan_kernel<NRv, DTv><<<grid, 256, 0, stream>>>(xbc, ldx, (const DTv*)dt, lddt, dt_bias, A_log, Dskip, state, \
-                                                        y, cu_q, seq_slot, heads, P, N, groups, write_state)
-#define BY_NR(DTv)                          \
-    do {                                    \
-        if (need <= 2) LAUNCH(2, DTv);      \
-        else if (need <= 4) LAUNCH(4, DTv); \
-        else if (need <= 8) LAUNCH(8, DTv); \
-        else if (need <= 16) LAUNCH(16, DTv); \
-        else LAUNCH(32, DTv);               \
+#define LAUNCH(NRv, TTv, DTv)                                                                                    \
+    ssm_scan_kernel<NRv, TTv, DTv><<<grid, 256, 0, stream>>>(xbc, ldx, (const DTv*)dt, lddt, dt_bias, A_log, Dskip, \
+                                                             state, y, cu_q, seq_slot, heads, P, N, groups, write_state)
+#define BY_NR(DTv)                                \
+    do {                                          \
+        if (need <= 2) LAUNCH(2, 32, DTv);        \
+        else if (need <= 4) LAUNCH(4, 32, DTv);   \
+        else if (need <= 8) LAUNCH(8, 32, DTv);   \
+        else if (need <= 16) LAUNCH(16, 32, DTv); \
+        else LAUNCH(32, 16, DTv);                 \
     } while (0)
     if (dt_dtype == CPMCU_F32) BY_NR(float);
     else if (dt_dtype == CPMCU_BF16) BY_NR(bf16_t);

@@ -1048,8 +1048,9 @@ def attention_general_mfma_ok(q: torch.Tensor, hdk: int, hdv: int, page_size: in
 
 
 def attention_general_splits(n_tokens: int, nkv: int, group: int, pool_hdv: int, max_keys: int) -> int:
-    """Shares of a token's keys for attention_general_mfma in steps of few tokens: as attention_splits says, and
-    four times as many where a workgroup is one wavefront (values too wide for its four to merge through LDS)."""
+    """Shares of a token's keys for attention_general_mfma in steps of few tokens: as attention_splits says (about
+    one workgroup a CU, a share of at least 128 keys); four times as many, of at least 64 keys, for values wider
+    than 128 features, whose workgroups do not split the keys among their wavefronts and so have less in flight."""
     s = attention_splits(n_tokens, nkv, group, max_keys)
     if pool_hdv > 128 and n_tokens <= compute_units():
         s = max(1, min(s * 4, 64, max_keys // 64))

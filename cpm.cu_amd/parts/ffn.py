@@ -64,7 +64,10 @@ class PolyNormFFN(FeedForward):
 
     def forward(self, h: torch.Tensor, ctx: StepContext):
         with ctx.timed("ffn_up"):
-            z = self.up.forward(h, ctx, "ffn.up", partials=True)
+            # few rows: float out of the decode product (one slice: its many output rows fill the chip without a
+            # split of K); many rows: the library's product in the engine's element type
+            few = h.shape[0] <= ops.SKINNY_MAX_ROWS
+            z = self.up.forward(h, ctx, "ffn.up", out_dtype=torch.float32 if few else None)
         act = ctx.ws.get("ffn.act", (h.shape[0], self.intermediate_size), self.rt.dtype)
         with ctx.timed("ffn_act"):
             ops.poly_norm(z, self.coef, self.eps, act)

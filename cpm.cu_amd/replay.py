@@ -29,7 +29,7 @@ def main(argv=None) -> int:
                     help="bfloat16: the kernels and precisions that serving uses; float32: everything in true 32-bit")
     ap.add_argument("--out", required=True, help="folder for <step>.f32 files")
     ap.add_argument("--max-tokens", type=int, required=True,
-                    help="most tokens that live requests hold at any time (each rounded up to 64); sizes the cache")
+                    help="most tokens that live requests hold at any time; sizes the cache")
     ap.add_argument("--max-step-tokens", type=int, default=2048, help="tokens one forward pass carries")
     ap.add_argument("--device", default="cuda:0")
     args = ap.parse_args(argv)
@@ -39,7 +39,12 @@ def main(argv=None) -> int:
 
     os.makedirs(args.out, exist_ok=True)
     print(f"[trace_run] loading {args.model} ({args.dtype})", file=sys.stderr, flush=True)
-    engine = Engine.from_dir(args.model, EngineOptions(dtype=args.dtype, max_tokens=max(args.max_tokens, 64),
+    # --max-tokens counts tokens, the cache holds whole pages: every live request may leave most of its last page
+    # empty, so the cache gets a page of slack for each of up to 64 requests
+    page = EngineOptions().page_size
+    tokens = max(args.max_tokens, 1)
+    engine = Engine.from_dir(args.model, EngineOptions(dtype=args.dtype, max_tokens=-(-tokens // page) * page + 64 * page,
+                                                       max_seq_len=-(-tokens // page) * page,
                                                        max_step_tokens=args.max_step_tokens, device=args.device))
     slots: Dict[str, int] = {}
     for line in sys.stdin:
