@@ -44,7 +44,6 @@ def main(argv=None) -> int:
     page = EngineOptions().page_size
     tokens = max(args.max_tokens, 1)
     engine = Engine.from_dir(args.model, EngineOptions(dtype=args.dtype, max_tokens=-(-tokens // page) * page + 64 * page,
-                                                       max_seq_len=-(-tokens // page) * page,
                                                        max_step_tokens=args.max_step_tokens, device=args.device))
     slots: Dict[str, int] = {}
     for line in sys.stdin:
