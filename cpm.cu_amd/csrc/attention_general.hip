@@ -210,21 +210,30 @@ __global__ __launch_bounds__(NW * TW * 64) void attention_general_mfma_kernel(
     const bf16_t* __restrict__ q, bf16_t* __restrict__ out, float* __restrict__ part_o, float2* __restrict__ part_ml,
     const bf16_t* __restrict__ kpool, const bf16_t* __restrict__ vtpool, PagedView pv,
     const int* __restrict__ positions, const int* __restrict__ tok_slot, int nh, int nkv, int hdk, int hdv,
-    int pool_hdk, int pool_hdv, float scale_log2e, int chunk, int n_splits, int n_tokens) {
+    int pool_hdk, int pool_hdv, float scale_log2e, int chunk, int n_splits, int n_tokens, const int* __restrict__ tiles,
+    int n_tiles, int tpt, int rpt) {
     extern __shared__ __align__(16) unsigned char smem[];
     static_assert(NW == 1 || TW == 1, "either the wavefronts of a workgroup share a token or each has its own");
     const int ksteps = (pool_hdk + 31) >> 5, dtn = pool_hdv >> 4;
     const int kvh = blockIdx.y % nkv, ht = blockIdx.y / nkv, split = blockIdx.z;
     const int wave_id = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
     const int wave = TW > 1 ? 0 : wave_id;
-    int t = blockIdx.x * TW + (TW > 1 ? wave_id : 0);
-    const bool live = t < n_tokens;
-    if (!live) t = n_tokens - 1;
+    // A wavefront's tile of 16 columns holds one token's heads, or (tiles given, groups smaller than 16) the
+    // heads of up to tpt consecutive tokens of one sequence, rpt columns each: column n is token n / rpt of
+    // the tile, head n % rpt of the group.
+    const int unit = blockIdx.x * TW + (TW > 1 ? wave_id : 0);
+    const int n_units = tiles ? n_tiles : n_tokens;
+    const bool live = unit < n_units;
+    const int un = live ? unit : n_units - 1;
+    const int t0 = tiles ? tiles[2 * un] : un, n_tok = tiles ? tiles[2 * un + 1] : 1;
     const int lane = threadIdx.x & 63, n = lane & 15, g = lane >> 4;
     const int G = nh / nkv;
-    const int head = kvh * G + ht * 16 + n;
-    const bool head_ok = ht * 16 + n < G;
-    const int pos = positions[t], slot = tok_slot[t];
+    const int tk = n / rpt, hh = ht * 16 + n % rpt;
+    const bool head_ok = tk < n_tok && tk < tpt && hh < G;
+    const int t = t0 + (tk < n_tok ? tk : 0);
+    const int head = kvh * G + (hh < G ? hh : 0);
+    const int pos = positions[t], slot = tok_slot[t0];
+    const int pos_min = positions[t0], pos_max = pos_min + n_tok - 1;     // a tile's tokens are consecutive
 
     // Q^T fragments of this wavefront's token: [ksteps][lane] of 8 features
     gbf16x8_t* qs = (gbf16x8_t*)smem + (long)(TW > 1 ? wave_id : 0) * ksteps * 64;
@@ -237,8 +246,9 @@ __global__ __launch_bounds__(NW * TW * 64) void attention_general_mfma_kernel(
     __syncthreads();
 
     const int first_key = chunk > 0 ? pos - pos % chunk : 0;
-    const int cfirst = first_key >> 5;
-    const int total_chunks = (pos >> 5) + 1 - cfirst;
+    const int first_min = chunk > 0 ? pos_min - pos_min % chunk : 0, first_max = chunk > 0 ? pos_max - pos_max % chunk : 0;
+    const int cfirst = first_min >> 5;
+    const int total_chunks = (pos_max >> 5) + 1 - cfirst;
     const int per_split = (total_chunks + n_splits - 1) / n_splits;
     const int c0 = split * per_split, c1 = min(c0 + per_split, total_chunks);
 
@@ -304,7 +314,7 @@ __global__ __launch_bounds__(NW * TW * 64) void attention_general_mfma_kernel(
             }
         }
         // lane (head n, g): st0[e] is key key0 + 8g + e, st1[e] is key key0 + 8g + 4 + e
-        if (key0 + 31 > pos || key0 < first_key) {
+        if (key0 + 31 > pos_min || key0 < first_max) {
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
                 const int ka = key0 + 8 * g + e, kb = ka + 4;
@@ -442,6 +452,7 @@ extern "C" const char* cpmcu_attention_general_mfma(const void* q, void* out, fl
                                                     float scale, int chunk, const void* kpool, const void* vtpool,
                                                     const int* page_table, int table_width, int page_size,
                                                     const int* positions, const int* tok_slot, int n_splits,
+                                                    const int* tiles, int n_tiles, int tokens_per_tile,
                                                     hipStream_t stream) {
     CPMCU_REQUIRE(n > 0 && nh > 0 && nkv > 0 && nh % nkv == 0, "attention_general_mfma: bad shape n=%d heads=%d kv_heads=%d", n, nh, nkv);
     CPMCU_REQUIRE(hdk > 0 && hdk % 8 == 0 && hdk <= 1024 && hdv > 0 && hdv <= 512,
@@ -466,15 +477,21 @@ extern "C" const char* cpmcu_attention_general_mfma(const void* q, void* out, fl
     // (four wavefronts that merge through LDS need room there beside the Q fragments)
     const long merge_bytes = (4 * 16 * 2 + 4L * dtm * 4 * 64) * 4;
     const int nw = (vs || (n <= 256 && q_bytes + merge_bytes <= 64 * 1024)) ? 4 : 1;
+    // tiles that pack several tokens: only where a wavefront has a tile to itself and nothing is merged
+    const int rpt = G < 16 ? G : 16;
+    CPMCU_REQUIRE(!tiles || (n_tiles > 0 && nw == 1 && n_splits == 1 && tokens_per_tile >= 1 && tokens_per_tile * rpt <= 16),
+                  "attention_general_mfma: tiles of %d tokens do not suit this step", tokens_per_tile);
+    const int tpt = tiles ? tokens_per_tile : 1;
+    const int units = tiles ? n_tiles : n;
     const int tw = (nw == 1 && n_splits == 1 && n >= 64 && 4 * q_bytes <= 48 * 1024) ? 4 : 1;
     const long lds = (tw > 1 ? tw * q_bytes : q_bytes) + ((nw > 1 && !vs) ? (nw * 16 * 2 + (long)nw * dtm * 4 * 64) * 4 : 0) +
                      (vs ? 2L * nw * 8 * 64 * 4 : 0);
     CPMCU_REQUIRE(lds <= 64 * 1024, "attention_general_mfma: %ld bytes of LDS", lds);
-    dim3 grid((n + tw - 1) / tw, nkv * HT, n_splits);
+    dim3 grid((units + tw - 1) / tw, nkv * HT, n_splits);
 #define LAUNCH(DTMv, NWv, TWv, VSv)                                                                              \
     attention_general_mfma_kernel<DTMv, NWv, TWv, VSv><<<grid, NWv * TWv * 64, lds, stream>>>(                   \
         (const bf16_t*)q, (bf16_t*)out, part_o, (float2*)part_ml, (const bf16_t*)kpool, (const bf16_t*)vtpool, pv, \
-        positions, tok_slot, nh, nkv, hdk, hdv, pool_hdk, pool_hdv, sl, chunk, n_splits, n)
+        positions, tok_slot, nh, nkv, hdk, hdv, pool_hdk, pool_hdv, sl, chunk, n_splits, n, tiles, n_tiles, tpt, rpt)
     if (vs) {
         if (dtm == 4) LAUNCH(4, 4, 1, true);
         else LAUNCH(8, 4, 1, true);

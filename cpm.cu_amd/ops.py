@@ -1060,10 +1060,14 @@ def attention_general_splits(n_tokens: int, nkv: int, group: int, pool_hdv: int,
 def attention_general_mfma(q: torch.Tensor, out: torch.Tensor, nh: int, nkv: int, hdk: int, hdv: int, scale: float,
                            kpool: torch.Tensor, vpool: torch.Tensor, page_table: torch.Tensor, page_size: int,
                            positions: torch.Tensor, tok_slot: torch.Tensor, chunk: int = 0, n_splits: int = 1,
-                           part_o: Optional[torch.Tensor] = None, part_ml: Optional[torch.Tensor] = None):
+                           part_o: Optional[torch.Tensor] = None, part_ml: Optional[torch.Tensor] = None,
+                           tiles: Optional[torch.Tensor] = None, tokens_per_tile: int = 1):
     """attention_general in bf16 on the matrix cores (key size a multiple of 8 up to 1024, value size up to 512).
     With n_splits > 1 every token's visible keys are shared among n_splits workgroups and merged afterwards;
-    part_o float32 [n, nh, n_splits, hdv] and part_ml float32 [n, nh, n_splits, 2] are its scratch."""
+    part_o float32 [n, nh, n_splits, hdv] and part_ml float32 [n, nh, n_splits, 2] are its scratch.
+    tiles (int32 [T, 2] = first packed token, tokens; prompts of more than 256 tokens with fewer than 16 heads a
+    kv head and values up to 128 features): runs of at most tokens_per_tile consecutive tokens of one sequence,
+    which share a matrix-core tile (tokens_per_tile * heads a kv head <= 16)."""
     _need(q, "attention q", torch.bfloat16, (None, nh * hdk))
     n = q.shape[0]
     _need(out, "attention out", torch.bfloat16, (n, nh * hdv))
@@ -1077,11 +1081,23 @@ def attention_general_mfma(q: torch.Tensor, out: torch.Tensor, nh: int, nkv: int
     if n_splits > 1:
         _need(part_o, "attention partial outputs", torch.float32, (n, nh, n_splits, hdv))
         _need(part_ml, "attention partial max/sum", torch.float32, (n, nh, n_splits, 2))
+    if tiles is not None:
+        _need(tiles, "attention tiles", torch.int32, (None, 2))
     _check(_fn("attention_general", "cpmcu_attention_general_mfma")(
         _p(q), _p(out), _p(part_o), _p(part_ml), c_int(n), c_int(nh), c_int(nkv), c_int(hdk), c_int(hdv),
         c_int(kpool.shape[2] // nkv), c_int(vpool.shape[2] // nkv), c_float(scale), c_int(chunk), _p(kpool), _p(vpool),
         _p(page_table), c_int(page_table.shape[1]), c_int(page_size), _p(positions), _p(tok_slot), c_int(n_splits),
-        _stream()))
+        _p(tiles), c_int(tiles.shape[0] if tiles is not None else 0), c_int(tokens_per_tile), _stream()))
+
+
+def attention_general_tokens_per_tile(n_tokens: int, nh: int, nkv: int, pool_hdv: int) -> int:
+    """Tokens that share a matrix-core tile in attention_general_mfma: prompts of more than 256 tokens whose
+    kv heads serve fewer than 16 query heads (and whose values a wavefront holds alone) fill the tile's 16
+    columns with the heads of several consecutive tokens; 1 everywhere else."""
+    group = nh // nkv
+    if n_tokens <= 256 or pool_hdv > 128 or group > 8:
+        return 1
+    return 16 // group
 
 
 def reserve_attention_general(ws, dtype, nh: int, nkv: int, hdv: int, pool_hdv: int, max_keys: int, max_step_tokens: int):
@@ -1110,8 +1126,16 @@ def attention_any(q, out, nh, nkv, hdk, hdv, scale, kpool, vpool, page_table, pa
         if splits > 1:
             part_o = ctx.ws.get("attn.gpart_o", (n, nh, splits, hdv), torch.float32)
             part_ml = ctx.ws.get("attn.gpart_ml", (n, nh, splits, 2), torch.float32)
+        tiles, tpt = None, 1
+        if not ctx.single_token:
+            tpt = attention_general_tokens_per_tile(n, nh, nkv, vpool.shape[2] // nkv)
+            if tpt > 1:
+                key = ("prefill_tiles", tpt)
+                tiles = ctx.extras.get(key)
+                if tiles is None:
+                    tiles = ctx.extras[key] = prefill_tiles(ctx.q_lens, tpt, q.device)
         attention_general_mfma(q, out, nh, nkv, hdk, hdv, scale, kpool, vpool, page_table, page_size, ctx.positions,
-                               ctx.tok_slot, chunk, splits, part_o, part_ml)
+                               ctx.tok_slot, chunk, splits, part_o, part_ml, tiles, tpt)
         return
     attention_general(q, out, nh, nkv, hdk, hdv, scale, kpool, vpool, page_table, page_size, ctx.positions,
                       ctx.tok_slot, chunk)

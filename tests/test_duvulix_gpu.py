@@ -203,3 +203,52 @@ def test_generation_loop_with_unequal_requests(models):
         assert list(o.tokens) == plain.greedy(cfg, w, p, 12)
     eng.cache.check()
     assert not eng.cache.live
+
+
+def test_replay_program_with_a_tight_token_budget(models, tmp_path):
+    """bin/trace_run as a user runs it (float32): an unequal batch whose requests leave their last pages mostly
+    empty, with --max-tokens the bare sum of their tokens; then a request that takes freed slots and pages."""
+    import json
+    import os
+    import subprocess
+    import sys
+
+    import numpy as np
+    d, cfg, w, reqs, refs = models["Q"]
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    names = ["b", "c", "a", "f"]
+    prompt = {"b": 160, "c": 66, "a": 2, "f": 1}
+    steps = [{"step": 0, "entries": [{"id": r, "tokens": reqs[r][:prompt[r]], "want": [0, prompt[r] - 1]} for r in names],
+              "end": ["f"]}]
+    fed = dict(prompt)
+    fed["f"] = LENS["f"]
+    n = 1
+    while any(fed[r] < LENS[r] for r in names):
+        live = [r for r in names if fed[r] < LENS[r]]
+        steps.append({"step": n, "entries": [{"id": r, "tokens": [reqs[r][fed[r]]], "want": [0]} for r in live],
+                      "end": [r for r in live if fed[r] + 1 == LENS[r]]})
+        for r in live:
+            fed[r] += 1
+        n += 1
+    steps.append({"step": n, "entries": [{"id": "again", "tokens": reqs["d"], "want": [LENS["d"] - 1]}], "end": ["again"]})
+    out = tmp_path / "out"
+    budget = LENS["b"] + LENS["c"] + LENS["a"] + 1
+    proc = subprocess.run([sys.executable, os.path.join(root, "bin", "trace_run"), "--model", d, "--dtype", "float32",
+                           "--out", str(out), "--max-tokens", str(budget)],
+                          input="".join(json.dumps(s) + "\n" for s in steps), capture_output=True, text=True, timeout=600)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    assert [l for l in proc.stdout.split("\n") if l.startswith("done")] == [f"done {s['step']}" for s in steps]
+    V = cfg["vocab"]
+    at = dict(prompt)
+    for s in steps[:-1]:
+        rows = []
+        for e in s["entries"]:
+            base = 0 if s["step"] == 0 else at[e["id"]]
+            rows += [refs[e["id"]][base + wpos] for wpos in e["want"]]
+        if s["step"] > 0:
+            for e in s["entries"]:
+                at[e["id"]] += 1
+        got = torch.from_numpy(np.fromfile(out / f"{s['step']}.f32", dtype="<f4").reshape(len(rows), V))
+        assert float((got - torch.stack(rows)).abs().max()) < 1e-4, f"step {s['step']}"
+    got = torch.from_numpy(np.fromfile(out / f"{n}.f32", dtype="<f4").reshape(1, V))
+    assert float((got[0] - refs["d"][-1]).abs().max()) < 1e-4

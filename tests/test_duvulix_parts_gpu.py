@@ -244,6 +244,49 @@ def test_matrix_core_attention_against_the_plain_kernel_and_the_plain_implementa
         close(out, want[a:b], "bfloat16")
 
 
+@pytest.mark.parametrize("shape", [(8, 2, 48, 32, 40), (6, 1, 64, 64, 33), (4, 4, 32, 96, 0), (5, 1, 40, 24, 100)])
+def test_matrix_core_attention_with_several_tokens_a_tile(shape):
+    """Prompts of more than 256 tokens whose kv heads serve few query heads: consecutive tokens of one sequence
+    share a tile.  Two sequences of unequal length in one packed batch, the second continuing from cached
+    tokens; runs never straddle the sequences."""
+    from cpmcu_amd import ops
+    H, G, dk, dv, chunk = shape
+    torch.manual_seed(17)
+    page, T1, T2, old2 = 64, 301, 140, 37                 # sequence 2 holds 37 tokens already
+    L2 = old2 + T2
+    k = [torch.randn(T1, G, dk).to(torch.bfloat16), torch.randn(L2, G, dk).to(torch.bfloat16)]
+    v = [torch.randn(T1, G, dv).to(torch.bfloat16), torch.randn(L2, G, dv).to(torch.bfloat16)]
+    q = [torch.randn(T1, H, dk).to(torch.bfloat16), torch.randn(L2, H, dk).to(torch.bfloat16)]
+    pk, pv = -(-dk // 16) * 16, -(-dv // 16) * 16
+    kp = torch.zeros(12, page, G * pk, dtype=torch.bfloat16, device=DEV)
+    vp = torch.zeros(12, page, G * pv, dtype=torch.bfloat16, device=DEV)
+    table = torch.zeros(3, 5, dtype=torch.int32)
+    table[2, :5] = torch.tensor([3, 9, 0, 7, 5])
+    table[0, :3] = torch.tensor([11, 1, 6])
+    table = dev(table)
+    for sl, kk, vv in ((2, k[0], v[0]), (0, k[1], v[1])):
+        Tn = kk.shape[0]
+        paged = dict(tok_slot=dev(torch.full((Tn,), sl, dtype=torch.int32)), page_table=table, page_size=page, pool_heads=G)
+        pos = dev(torch.arange(Tn, dtype=torch.int32))
+        ops.rotate_copy(dev(kk.reshape(Tn, G * dk)), 0, dk, G, dk, 0, pos, None, 1.0, kp, ops.ROTATE_TO_KEYS, pool_hd=pk, **paged)
+        ops.rotate_copy(dev(vv.reshape(Tn, G * dv)), 0, dv, G, dv, 0, pos, None, 1.0, vp, ops.ROTATE_TO_VALUES, pool_hd=pv, **paged)
+    want = []
+    for i in range(2):
+        s = torch.einsum("ihd,jhd->hij", q[i].double(), k[i].double().repeat_interleave(H // G, 1)) * 0.2
+        want.append(plain.softmax_attend(s, plain.visible(q[i].shape[0], chunk or None),
+                                         v[i].double().repeat_interleave(H // G, 1)).reshape(-1, H * dv))
+    qd = dev(torch.cat([q[0], q[1][old2:]]).reshape(T1 + T2, H * dk))
+    pos = dev(torch.cat([torch.arange(T1), torch.arange(old2, L2)]).to(torch.int32))
+    slot = dev(torch.cat([torch.full((T1,), 2), torch.full((T2,), 0)]).to(torch.int32))
+    tpt = ops.attention_general_tokens_per_tile(T1 + T2, H, G, pv)
+    assert tpt == 16 // (H // G)
+    tiles = ops.prefill_tiles([T1, T2], tpt, DEV)
+    out = torch.empty(T1 + T2, H * dv, dtype=torch.bfloat16, device=DEV)
+    ops.attention_general_mfma(qd, out, H, G, dk, dv, 0.2, kp, vp, table, page, pos, slot, chunk, tiles=tiles,
+                               tokens_per_tile=tpt)
+    close(out, torch.cat([want[0], want[1][old2:]]), "bfloat16")
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_one_key_that_stands_out_at_the_edges_of_a_chunk(dtype):
     """The key at one position is made to dominate every query.  A query sees it exactly when it lies in the
