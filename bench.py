@@ -173,7 +173,7 @@ def main():
                     help="after the timed runs, a few eager steps with the engine's timers on: average ms by kernel "
                          "class (products / attention / selection / norms / head) on stderr and under 'timers'")
     ap.add_argument("--scenario", default="headline", choices=["headline", "small_batch64", "sparse32k", "duvulix"],
-                    help="headline: the 8B shape at batch 8, context 4,096 (the default, the contract's line); "
+                    help="headline: the 8B shape at batch 8, context 4,096 (the default line); "
                          "small_batch64: the 0.5B shape, 64 unequal prompts through the generation loop; sparse32k: "
                          "the 8B shape with InfLLM-v2 at 32k context; duvulix: four Duvulix layers of a real model's "
                          "sizes (latent attention, chunked attention, Mamba-2, a layer that reads the first one's "

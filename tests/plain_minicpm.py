@@ -3,7 +3,7 @@
 Whole sequences, no cache, one function per part, written from the formulas of
 OpenBMB/CPM.cu (cited per function as path:line of that repository) and, where
 that engine holds one sequence or leaves a choice open, from the engine's own
-contract (block-sparse attention as a pure function of the prefix).  It shares
+definition (block-sparse attention as a pure function of the prefix).  It shares
 no code with the product package: it only needs torch on the CPU, a raw
 config.json dict and a dict of tensors by their checkpoint names.
 
