@@ -252,3 +252,43 @@ def test_replay_program_with_a_tight_token_budget(models, tmp_path):
         assert float((got - torch.stack(rows)).abs().max()) < 1e-4, f"step {s['step']}"
     got = torch.from_numpy(np.fromfile(out / f"{n}.f32", dtype="<f4").reshape(1, V))
     assert float((got[0] - refs["d"][-1]).abs().max()) < 1e-4
+
+
+def test_command_line(models, tmp_path):
+    """The command line on a Duvulix folder (greedy tokens equal the plain implementation's, the timers name the
+    new kernel classes), with sampling, and in random-weights mode from a config.json alone."""
+    import json
+    import os
+    import subprocess
+    import sys
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+    def run_cli(*args):
+        env = dict(os.environ, PYTHONPATH=root)
+        return subprocess.run([sys.executable, "-m", "cpmcu_amd.cli", *args], capture_output=True, text=True,
+                              timeout=600, env=env)
+    d, cfg, w, reqs, refs = models["P"]
+    prompts = [reqs["a"][:6], reqs["c"][:45]]
+    ids = tmp_path / "ids.txt"
+    ids.write_text("\n".join(" ".join(map(str, p)) for p in prompts) + "\n")
+    p = run_cli("--model-path", d, "--dtype", "float32", "--prompt-ids", str(ids), "--num-generate", "6",
+                "--ignore-eos", "true", "--max-tokens", "512", "--use_stream", "false", "--perf")
+    assert p.returncode == 0, p.stderr[-1500:]
+    assert "prefill_ssm_scan" in p.stdout and "decode_attn_core" in p.stdout and "decode_ffn_act" in p.stdout
+    lines = [l for l in p.stdout.splitlines() if l.startswith("[")]
+    assert [[int(t) for t in l.split(") ")[1].split()] for l in lines] == [plain.greedy(cfg, w, pr, 6) for pr in prompts]
+    outs = []
+    for _ in range(2):
+        p = run_cli("--model", d, "--prompt-ids", str(ids), "--num_generate", "5", "--temperature", "0.8",
+                    "--random-seed", "11", "--max-tokens", "512", "--use-stream", "false")
+        assert p.returncode == 0, p.stderr[-1500:]
+        outs.append(p.stdout)
+    assert outs[0] == outs[1] and outs[0].strip()
+    cfgp = tmp_path / "config.json"
+    cfgp.write_text(json.dumps(td.tiny_q()))
+    out = tmp_path / "model"
+    p = run_cli("--random-weights", "--config", str(cfgp), "--seed", "3", "--model-path", str(out), "--prompt-lens", "70,5",
+                "--num-generate", "3", "--max-tokens", "512")
+    assert p.returncode == 0, p.stderr[-1500:]
+    assert sorted(os.listdir(out)) == ["config.json", "model.safetensors"]
+    assert len([l for l in p.stdout.splitlines() if l.startswith("[")]) == 2
