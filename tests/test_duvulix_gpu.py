@@ -21,7 +21,7 @@ BATCHES = [("a", "b", "c"), ("d", "e", "f"), ("c", "a"), ("f", "b", "d")]
 @pytest.fixture(scope="module")
 def models(tmp_path_factory):
     out = {}
-    for name, raw, seed in (("P", td.tiny_p(), 31), ("Q", td.tiny_q(), 47)):
+    for name, raw, seed in (("P", td.tiny_p(), 31), ("Q", td.tiny_q(), 47), ("R", td.tiny_r(), 59)):
         d = str(tmp_path_factory.mktemp(f"duvulix_{name}"))
         td.write_model(raw, d, seed)
         cfg, w = tiny.read_model(d)
@@ -73,6 +73,20 @@ def test_whole_prompts(models, name, dtype):
     check(schedules.whole(eng, reqs), refs, dtype, "whole")
     eng.cache.check()
     assert not eng.cache.live
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_sizes_that_suit_no_tuned_kernel(models, dtype):
+    """A width of 100, heads of 20 and 12 features, a latent of 36, a state of 7: every dispatcher falls back to
+    its plain kernel where the tuned one does not take the size, and the results are the same."""
+    _, cfg, w, reqs, refs = models["R"]
+    eng = engine_for(models, "R", dtype)
+    check(schedules.whole(eng, reqs), refs, dtype, "whole, odd sizes")
+    check(schedules.tail(eng, reqs, 45), refs, dtype, "tail-45, odd sizes")
+    used = ("a", "b", "c")
+    got = schedules.batched(eng, {r: reqs[r] for r in used}, PROMPT, [used])
+    check(got, {r: refs[r] for r in used}, dtype, "batched, odd sizes")
+    eng.cache.check()
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])

@@ -52,6 +52,28 @@ def tiny_q():
     }
 
 
+def tiny_r():
+    """Sizes that suit no vector access and no matrix-core tile: a width of 100, a vocabulary of 77, heads of 20 and
+    12 features, a latent of 36 with 4 rotated features, 5 kv heads of 3 query heads each, a state of 7."""
+    return {
+        "architecture": "Duvulix", "vocab": 77, "width": 100, "norm": {"eps": 1e-6},
+        "layers": [
+            {"type": "attention", "mixer": {"heads": 15, "kv_heads": 5, "dim": 20, "vdim": 12, "scale": 0.3,
+                                            "rot": {"base": 1000.0, "dims": 6}, "mask": {"size": 17}},
+             "mlp": {"kind": "dense", "ff": 52}},
+            {"type": "latent_attention", "mixer": {"heads": 3, "dim": 20, "rot_dim": 4, "vdim": 12, "kv_rank": 36,
+                                                   "scale": 0.25, "rot": {"base": 777.0, "dims": 4}},
+             "mlp": {"kind": "dense", "ff": 30}},
+            {"type": "mamba2", "mixer": {"heads": 3, "vdim": 5, "state": 7, "groups": 3, "conv": 2, "norm_groups": 5},
+             "mlp": None},
+            {"type": "attention", "mixer": {"heads": 2, "kv_heads": 1, "dim": 40, "vdim": 40, "scale": 0.2,
+                                            "rot": {"base": 1000.0, "dims": 40,
+                                                    "scaling": {"factor": 16.0, "original": 24, "fast": 8.0, "slow": 1.0}}},
+             "mlp": {"kind": "dense", "ff": 52}},
+        ],
+    }
+
+
 def write_model(raw, out_dir, seed, std=0.08, norm_std=0.1):
     """A model folder with random weights through the package's own writer; config.json is the raw dictionary."""
     import cpmcu_amd
