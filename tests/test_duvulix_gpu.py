@@ -306,3 +306,24 @@ def test_command_line(models, tmp_path):
     assert p.returncode == 0, p.stderr[-1500:]
     assert sorted(os.listdir(out)) == ["config.json", "model.safetensors"]
     assert len([l for l in p.stdout.splitlines() if l.startswith("[")]) == 2
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["P", "Q"])
+def test_a_long_sequence(models, name, dtype):
+    """1,300 tokens (21 pages, 32 chunks of the mask): the prompt in passes of 512 tokens, then 40 tokens one by
+    one, where the attention over more than a thousand cached tokens runs in shares that are merged and the
+    recurrent state has been carried through the whole prompt."""
+    from cpmcu_amd import StepEntry
+    _, cfg, w, reqs, refs = models[name]
+    toks = tiny.random_tokens(1300, cfg["vocab"], 900)
+    ref = plain.forward(cfg, w, toks).float()
+    eng = engine_for(models, name, dtype, max_tokens=2048, max_seq_len=1408, max_step_tokens=512)
+    s = eng.acquire()
+    want = list(range(0, 1260, 97)) + [1259]
+    got = [eng.step([StepEntry(s, toks[:1260], want)]).cpu()]
+    for i in range(1260, 1300):
+        got.append(eng.step([StepEntry(s, toks[i:i + 1], [0])]).cpu())
+    eng.release(s)
+    rows = want + list(range(1260, 1300))
+    check({"long": torch.cat(got)}, {"long": ref[rows]}, dtype, "a long sequence")
