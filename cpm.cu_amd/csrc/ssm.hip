@@ -3,7 +3,8 @@
 //  * conv_silu_kernel: causal convolution per channel over a sequence's tokens (taps weights a channel, the last
 //    column is the current token's; inputs before the sequence's start are zero) followed by SiLU.  The
 //    sequence's last taps-1 inputs live in the slot's state, so a step continues where the last one ended.
-//  * conv_state_kernel: moves the step's last inputs into that state (after the convolution has read it).
+//  * conv_state_kernel: moves the step's last inputs into that state (after the convolution has read it); for
+//    steps of at most 16 tokens a sequence the convolution's kernel does that itself.
 //  * ssm_scan_kernel: the recurrence, per head h (group g = h / (heads / groups)):
 //        dt_t = softplus(raw_t + dt_bias_h)             (no clamp)
 //        S_t  = exp(-exp(A_log_h) * dt_t) * S_(t-1) + dt_t * B_t x_t^T        S: [state N, head size P]
@@ -22,9 +23,9 @@ template <typename UT>
 __global__ __launch_bounds__(256) void conv_silu_kernel(const UT* __restrict__ u, long ldu,
                                                         const float* __restrict__ weight,
                                                         const float* __restrict__ bias,
-                                                        const float* __restrict__ state, float* __restrict__ out,
+                                                        const float* state, float* __restrict__ out,
                                                         const int* __restrict__ cu_q, const int* __restrict__ seq_slot,
-                                                        int C, int taps) {
+                                                        int C, int taps, float* state_out) {
     const int b = blockIdx.x;
     const int start = cu_q[b], q = cu_q[b + 1] - start;
     const int slot = seq_slot[b];
@@ -41,6 +42,15 @@ __global__ __launch_bounds__(256) void conv_silu_kernel(const UT* __restrict__ u
             acc += weight[(long)c * taps + k] * in;
         }
         out[(long)(start + i) * C + c] = silu_f(acc);
+    }
+    // steps of at most 16 tokens a sequence (decode steps): this thread alone has read its channel's state, so
+    // it moves the step's last inputs into it itself and the second kernel is not launched
+    if (state_out) {
+        float* so = state_out + (long)slot * (taps - 1) * C + c;
+        for (int j = 0; j < taps - 1; ++j) {
+            const int i = q - (taps - 1) + j;
+            so[(long)j * C] = i >= 0 ? to_f32(u[(long)(start + i) * ldu + c]) : so[(long)(j + q) * C];
+        }
     }
 }
 
@@ -74,13 +84,15 @@ extern "C" const char* cpmcu_conv_silu(const void* u, long ldu, int u_dtype, con
     CPMCU_REQUIRE(tb <= 65535 && cb <= 65535, "conv_silu: shape exceeds the launch grid (a step brings at most 1,048,560 "
                   "tokens a sequence)");
     dim3 grid(n_seqs, tb, cb), grid2(n_seqs, cb);
+    const bool moves = update_state && taps > 1;
+    float* fused = (moves && tb == 1) ? state : nullptr;
     if (u_dtype == CPMCU_F32) {
-        conv_silu_kernel<float><<<grid, 256, 0, stream>>>((const float*)u, ldu, weight, bias, state, out, cu_q, seq_slot, C, taps);
-        if (update_state && taps > 1)
+        conv_silu_kernel<float><<<grid, 256, 0, stream>>>((const float*)u, ldu, weight, bias, state, out, cu_q, seq_slot, C, taps, fused);
+        if (moves && !fused)
             conv_state_kernel<float><<<grid2, 256, 0, stream>>>((const float*)u, ldu, state, cu_q, seq_slot, C, taps);
     } else if (u_dtype == CPMCU_BF16) {
-        conv_silu_kernel<bf16_t><<<grid, 256, 0, stream>>>((const bf16_t*)u, ldu, weight, bias, state, out, cu_q, seq_slot, C, taps);
-        if (update_state && taps > 1)
+        conv_silu_kernel<bf16_t><<<grid, 256, 0, stream>>>((const bf16_t*)u, ldu, weight, bias, state, out, cu_q, seq_slot, C, taps, fused);
+        if (moves && !fused)
             conv_state_kernel<bf16_t><<<grid2, 256, 0, stream>>>((const bf16_t*)u, ldu, state, cu_q, seq_slot, C, taps);
     } else {
         CPMCU_FAIL("conv_silu: unknown dtype %d", u_dtype);
