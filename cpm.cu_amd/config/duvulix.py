@@ -95,7 +95,9 @@ class AttentionConfig:
         g = lambda k: field_from(raw, k, int, where=where)
         mask = raw.get("mask")
         require(mask is None or isinstance(mask, dict), f"{where}: 'mask' must be an object")
-        c = cls(g("heads"), g("kv_heads"), g("dim"), g("vdim"), field_from(raw, "scale", float, where=where),
+        # a configuration that leaves these out means the plain case: a kv head a head, values as wide as keys
+        c = cls(g("heads"), field_from(raw, "kv_heads", int, g("heads"), where=where), g("dim"),
+                field_from(raw, "vdim", int, g("dim"), where=where), field_from(raw, "scale", float, where=where),
                 Rotation.from_dict(raw.get("rot"), where),
                 field_from(mask, "size", int, where=where + " mask") if mask is not None else None)
         require(min(c.heads, c.kv_heads, c.dim, c.vdim) > 0, f"{where}: sizes must be positive")
@@ -123,7 +125,9 @@ class Mamba2Config:
 
     @classmethod
     def from_dict(cls, raw: Dict[str, Any], where: str):
-        c = cls(*(field_from(raw, k, int, where=where) for k in ("heads", "vdim", "state", "groups", "conv", "norm_groups")))
+        c = cls(field_from(raw, "heads", int, where=where), field_from(raw, "vdim", int, where=where),
+                field_from(raw, "state", int, where=where), field_from(raw, "groups", int, 1, where=where),
+                field_from(raw, "conv", int, where=where), field_from(raw, "norm_groups", int, 1, where=where))
         require(min(c.heads, c.vdim, c.state, c.groups, c.conv, c.norm_groups) > 0, f"{where}: sizes must be positive")
         require(c.heads % c.groups == 0, f"{where}: heads ({c.heads}) must be a multiple of groups ({c.groups})")
         require((c.heads * c.vdim) % c.norm_groups == 0,

@@ -94,7 +94,7 @@ def test_yarn_frequencies_of_the_part_equal_the_plain_ones():
     from cpmcu_amd.parts.base import Runtime, Workspace
     rt = Runtime(torch.device("cpu"), torch.float32, Workspace("cpu"), 256)
     for rot in ({"base": 10000.0, "dims": 32, "scaling": {"factor": 4.0, "original": 64, "fast": 16.0, "slow": 2.0}},
-                {"base": 20000.0, "dims": 96, "scaling": {"factor": 2.0, "original": 4096, "fast": 32.0, "slow": 1.0}},
+                {"base": 250000.0, "dims": 128, "scaling": {"factor": 8.0, "original": 8192, "fast": 24.0, "slow": 0.5}},
                 {"base": 500.0, "dims": 8, "scaling": {"factor": 8.0, "original": 32, "fast": 1.0, "slow": 1.0}}):
         sc = rot["scaling"]
         enc = POSITION_ENCODINGS.build("yarn", head_dim=rot["dims"], theta=rot["base"], factor=sc["factor"],
