@@ -394,7 +394,11 @@ class Engine:
         graph = self.uses_graph
         rows = np.arange(B, dtype=np.int32) if graph else np.asarray(want_rows, dtype=np.int32)
         host = np.concatenate([tok.astype(np.int32), pos, sl, np.arange(B + 1, dtype=np.int32), sl, pos + 1, rows])
-        state = cache.snapshot_state(slots)
+        # A step that replays a captured graph launches nothing from the host that could refuse its arguments: it
+        # runs as a whole or the device itself has failed, so the copy of the slots' fixed-size state that a
+        # roll-back would put back is not made (for a model with recurrent layers it would read and write all of
+        # that state once more, every step).
+        state = None if self._replays(graph, B, int(pos.max())) else cache.snapshot_state(slots)
         try:
             logits = self._run(host, B, B, [1] * B, int(pos.max()), True, graph, int(rows.size), device_tokens)
         except BaseException:
@@ -406,6 +410,21 @@ class Engine:
             return logits.index_select(0, torch.tensor(want_rows, dtype=torch.long).to(self.device, non_blocking=True))
         return logits.clone()
 
+    def _graph_key(self, B: int, max_pos: int) -> Tuple[int, int]:
+        """A captured step sizes its launches for the largest position of a whole range of steps, so that one
+        capture serves all of them: the key is the batch size and that bound."""
+        bound = 256
+        while bound < max_pos + 1:
+            bound *= 2
+        return B, min(bound, self.max_seq_len) - 1
+
+    def _replays(self, graph: bool, B: int, max_pos: int) -> bool:
+        """Whether _run will replay a graph captured earlier for a step of this batch size and position."""
+        if not graph or (self.perf is not None and self.perf.enabled):
+            return False
+        entry = self._graphs.get(self._graph_key(B, max_pos))
+        return entry is not None and entry[3] == self.workspace.generation
+
     def _run(self, host: np.ndarray, n: int, B: int, q_lens: List[int], max_pos: int, single: bool, graph: bool,
              R: int, device_tokens: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
         """Upload one forward pass's metadata (tokens, positions, token slots, sequence starts, sequence slots,
@@ -414,12 +433,7 @@ class Engine:
         perf_on = self.perf is not None and self.perf.enabled
         graph = graph and not perf_on
         if graph:
-            # a captured step sizes its launches for the largest position of a whole range of steps, so that
-            # one capture serves all of them
-            bound = 256
-            while bound < max_pos + 1:
-                bound *= 2
-            max_pos = min(bound, self.max_seq_len) - 1
+            max_pos = self._graph_key(B, max_pos)[1]
         key = (B, max_pos)
         entry = self._graphs.get(key) if graph else None
         if entry is not None and entry[3] != self.workspace.generation:
