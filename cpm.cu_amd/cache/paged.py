@@ -50,9 +50,10 @@ class CacheNeeds:
     streams: Tuple[Tuple[str, StreamSpec], ...] = ()
     state: Tuple[Tuple[str, StateSpec], ...] = ()
     window: Optional[int] = None              # None: keep every token; w: only the last w tokens are read
+    keep_first: int = 0                       # with a window: the sequence's first tokens that stay readable for good
 
     def group_key(self):
-        return (self.streams, self.state, self.window)
+        return (self.streams, self.state, self.window, self.keep_first if self.window is not None else 0)
 
 
 @dataclass
@@ -63,6 +64,7 @@ class CacheView:
     page_table: Optional[torch.Tensor]        # int32 [max_slots, table_width] of the entry's group
     page_size: int
     window: Optional[int]
+    keep_first: int = 0
 
 
 class _Group:
@@ -72,6 +74,8 @@ class _Group:
         self.entries = entries
         self.n_pages = n_pages
         self.page_size = page_size
+        # pages at a sequence's start that a windowed group never gives back (they hold the tokens kept for good)
+        self.pinned = -(-needs.keep_first // page_size) if needs.window is not None else 0
         self.free_pages: List[int] = list(range(n_pages - 1, -1, -1))   # pop() gives the lowest page first
         # host page table: slot -> list of physical pages by page number (-1: given back / never held)
         self.pages: List[List[int]] = [[] for _ in range(max_slots)]
@@ -99,10 +103,11 @@ def _element_size(dtype: torch.dtype) -> int:
     return torch.empty((), dtype=dtype).element_size()
 
 
-def _window_pages(window: int, step: int, page_size: int) -> int:
+def _window_pages(window: int, step: int, page_size: int, keep_first: int = 0) -> int:
     """The most pages a sequence holds in a group that keeps a trailing window, when it grows by at most
-    ``step`` tokens at once: the step's first query still reads window - 1 tokens back."""
-    return (step + window - 2) // page_size + 2
+    ``step`` tokens at once: the step's first query still reads window - 1 tokens back.  The pages of the
+    first ``keep_first`` tokens are held beside them."""
+    return (step + window - 2) // page_size + 2 + -(-keep_first // page_size)
 
 
 def _pool_pages(needs: CacheNeeds, n_pages: int, max_slots: int, max_seq_len: int, step: int, page_size: int) -> int:
@@ -110,7 +115,7 @@ def _pool_pages(needs: CacheNeeds, n_pages: int, max_slots: int, max_seq_len: in
     holds; a group that keeps a window never holds more than its window's pages for every slot."""
     if needs.window is None:
         return n_pages
-    per_slot = min(-(-max_seq_len // page_size), _window_pages(needs.window, step, page_size))
+    per_slot = min(-(-max_seq_len // page_size), _window_pages(needs.window, step, page_size, needs.keep_first))
     return min(n_pages, max_slots * per_slot)
 
 
@@ -239,10 +244,11 @@ class SequenceCache:
         if g.needs.window is None:
             return max(n_pg - len(pages), 0), 0
         first_kept = self._first_kept(g, old)
-        need = max(n_pg - max(len(pages), first_kept), 0)
-        need += sum(1 for pn in range(first_kept, min(len(pages), n_pg)) if pages[pn] < 0)
+        pinned = g.pinned
+        need = max(n_pg - max(len(pages), first_kept, pinned), 0) + max(min(pinned, n_pg) - len(pages), 0)
+        need += sum(1 for pn in range(max(first_kept, pinned), min(len(pages), n_pg)) if pages[pn] < 0)
         freed = 0
-        for pn in range(min(first_kept, len(pages)) - 1, -1, -1):
+        for pn in range(min(first_kept, len(pages)) - 1, pinned - 1, -1):
             if pages[pn] < 0:
                 break
             freed += 1
@@ -256,11 +262,13 @@ class SequenceCache:
         for gi, g in enumerate(self.groups):
             free = len(g.free_pages)
             state: Dict[int, Tuple[int, int, int]] = {}        # slot -> (tokens, first held page number, page numbers)
+            pinned = g.pinned
             for one in passes:
                 for slot, n_new in one:
                     if slot not in state:
                         pages = g.pages[slot]
-                        lo = next((pn for pn, p in enumerate(pages) if p >= 0), len(pages))
+                        # the first page held behind the pinned ones (those are never given back)
+                        lo = next((pn for pn in range(min(pinned, len(pages)), len(pages)) if pages[pn] >= 0), len(pages))
                         state[slot] = (self.length(slot), lo, len(pages))
                     old, lo, hi = state[slot]
                     new = old + n_new
@@ -268,13 +276,14 @@ class SequenceCache:
                     lo2 = max(lo, first_kept)
                     free += max(min(lo2, hi) - lo, 0)                  # given back before anything is taken
                     hi2 = -(-new // self.page_size)
-                    need = max(hi2 - max(hi, first_kept), 0)
+                    need = max(hi2 - max(hi, first_kept, pinned), 0) + max(min(pinned, hi2) - hi, 0)
                     if need > free:
                         return (f"the cache is full: this step needs {need} more pages of {self.page_size} tokens"
                                 f"{'' if len(self.groups) == 1 else f' in cache group {gi}'} for slot {slot}, "
                                 f"{free} are free of {g.n_pages}")
                     free -= need
-                    state[slot] = (new, lo2, max(hi, hi2))
+                    hi3 = max(hi, hi2)
+                    state[slot] = (new, max(lo2, min(pinned, hi3)), hi3)
         return None
 
     def pages_to_hold(self, length: int, step: int) -> List[int]:
@@ -286,7 +295,7 @@ class SequenceCache:
             if g.needs.window is None:
                 out.append(full)
             else:
-                out.append(min(full, _window_pages(g.needs.window, step, self.page_size)))
+                out.append(min(full, _window_pages(g.needs.window, step, self.page_size, g.needs.keep_first)))
         return out
 
     def capacity(self) -> List[int]:
@@ -317,7 +326,7 @@ class SequenceCache:
             # the step's first query (position `old`) still reads back to old - window + 1
             first_kept = self._first_kept(g, old)
             changed = []
-            for pn in range(min(first_kept, len(pages)) - 1, -1, -1):
+            for pn in range(min(first_kept, len(pages)) - 1, g.pinned - 1, -1):
                 if pages[pn] < 0:
                     break                       # everything before an entry given back was given back earlier
                 g.free_pages.append(pages[pn])
@@ -325,7 +334,7 @@ class SequenceCache:
                 changed.append(pn)
             while len(pages) < n_pg:
                 pn = len(pages)
-                pages.append(g.free_pages.pop() if pn >= first_kept else -1)
+                pages.append(g.free_pages.pop() if (pn >= first_kept or pn < g.pinned) else -1)
                 changed.append(pn)
             if changed:
                 row = g.table_host[slot]
@@ -348,7 +357,7 @@ class SequenceCache:
             if g.needs.window is None:
                 continue
             pages = g.pages[slot]
-            gone = [pn for pn in range(self._first_kept(g, length), min(n_pg, len(pages))) if pages[pn] < 0]
+            gone = [pn for pn in range(max(self._first_kept(g, length), g.pinned), min(n_pg, len(pages))) if pages[pn] < 0]
             if gone:
                 raise CacheError(f"slot {slot}: cannot truncate to {length} tokens: cache group {gi} keeps a window of "
                                  f"{g.needs.window} tokens and has already given back page {gone[0]}, which the query "
@@ -405,7 +414,8 @@ class SequenceCache:
         v = self._views.get(entry)
         if v is None:
             g = self.groups[self.entry_group[entry]]
-            v = CacheView(g.storage[entry], g.state[entry], g.table, self.page_size, g.needs.window)
+            v = CacheView(g.storage[entry], g.state[entry], g.table, self.page_size, g.needs.window,
+                          g.needs.keep_first if g.needs.window is not None else 0)
             self._views[entry] = v
         return v
 

@@ -1,3 +1,4 @@
 from .base import ConfigError, ModelConfig, architecture_name, field_from, read_config_json, require
 from .minicpm import MiniCPMConfig, RopeScaling, SparseConfig
 from .duvulix import DuvulixConfig
+from .gumodra import GumodraConfig

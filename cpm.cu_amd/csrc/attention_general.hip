@@ -8,8 +8,10 @@
 //    rot_dims pass unchanged.
 //  * attention_general_kernel: the plain attention over the paged cache with key size hdk and value size hdv
 //    of their own (the cache may hold them padded to pool_hdk, pool_hdv), grouped heads, and an optional chunked mask: the query at position p sees keys j <= p with
-//    floor(j / chunk) == floor(p / chunk), chunks counted from position 0 of the sequence.  Float scores and
-//    softmax, both element types; one wavefront a (token, head).
+//    floor(j / chunk) == floor(p / chunk), chunks counted from position 0 of the sequence; or a sliding window
+//    with kept first tokens: key j <= p is seen if p - j < window or j < keep_first.  With `sink` (a float a head)
+//    the softmax's denominator holds exp(sink[head]) as one more term that has no key and no value.  Float scores
+//    and softmax, both element types; one wavefront a (token, head).
 //
 // Keys and values lie in their pages as common.h says (key_index, value_index), each with its own head size.
 #include "common.h"
@@ -98,7 +100,8 @@ template <typename T>
 __global__ __launch_bounds__(64) void attention_general_kernel(
     const T* __restrict__ q, T* __restrict__ out, const T* __restrict__ kpool, const T* __restrict__ vpool,
     PagedView pv, const int* __restrict__ positions, const int* __restrict__ tok_slot, int nh, int nkv, int hdk,
-    int hdv, int pool_hdk, int pool_hdv, float scale, int chunk) {
+    int hdv, int pool_hdk, int pool_hdv, float scale, int chunk, int window, int keep_first,
+    const float* __restrict__ sink) {
     __shared__ float qs[AG_MAX_HD];
     const int t = blockIdx.x, h = blockIdx.y, lane = threadIdx.x;
     const int g = h / (nh / nkv);
@@ -111,10 +114,13 @@ __global__ __launch_bounds__(64) void attention_general_kernel(
 #pragma unroll
     for (int i = 0; i < AG_MAX_HD / 64; ++i) acc[i] = 0.f;
     float m = -INFINITY, l = 0.f;
-    const int s0 = chunk > 0 ? pos - pos % chunk : 0, s1 = pos + 1;
-    for (int j0 = s0; j0 < s1; j0 += 64) {
-        const int j = j0 + lane;
-        const bool valid = j < s1;
+    const int s0 = chunk > 0 ? pos - pos % chunk : (window > 0 ? max(pos - window + 1, 0) : 0), s1 = pos + 1;
+    // the visible keys in one list: the kept first tokens that lie before the window, then the window
+    const int kept = min(keep_first, s0), total = kept + s1 - s0;
+    for (int i0 = 0; i0 < total; i0 += 64) {
+        const int i = i0 + lane;
+        const bool valid = i < total;
+        const int j = i < kept ? i : s0 + (i - kept);
         int row = 0;
         float s = -INFINITY;
         if (valid) {
@@ -129,7 +135,7 @@ __global__ __launch_bounds__(64) void attention_general_kernel(
         const float corr = expf(m - m_new);
         l = l * corr + wave_sum(p);
         m = m_new;
-        const int cnt = min(64, s1 - j0);
+        const int cnt = min(64, total - i0);
 #pragma unroll
         for (int i = 0; i < AG_MAX_HD / 64; ++i) acc[i] *= corr;
         for (int jj = 0; jj < cnt; ++jj) {
@@ -144,6 +150,7 @@ __global__ __launch_bounds__(64) void attention_general_kernel(
         }
     }
     T* orow = out + ((long)t * nh + h) * hdv;
+    if (sink) l += expf(sink[h] - m);
     const float inv = 1.0f / l;
 #pragma unroll
     for (int i = 0; i < AG_MAX_HD / 64; ++i) {
@@ -153,7 +160,8 @@ __global__ __launch_bounds__(64) void attention_general_kernel(
 }
 
 extern "C" const char* cpmcu_attention_general(const void* q, void* out, int dtype, int n, int nh, int nkv, int hdk,
-                                               int hdv, int pool_hdk, int pool_hdv, float scale, int chunk, const void* kpool,
+                                               int hdv, int pool_hdk, int pool_hdv, float scale, int chunk, int window,
+                                               int keep_first, const float* sink, const void* kpool,
                                                const void* vpool,
                                                const int* page_table, int table_width, int page_size,
                                                const int* positions, const int* tok_slot, hipStream_t stream) {
@@ -166,17 +174,21 @@ extern "C" const char* cpmcu_attention_general(const void* q, void* out, int dty
                   "attention_general: the cache holds heads in steps of 16 features and pages of a multiple of 32 tokens "
                   "(cached key size %d, value size %d, page %d)", pool_hdk, pool_hdv, page_size);
     CPMCU_REQUIRE(nh <= 65535, "attention_general: %d heads exceed the launch grid", nh);
-    CPMCU_REQUIRE(chunk >= 0, "attention_general: mask chunk %d", chunk);
+    CPMCU_REQUIRE(chunk >= 0 && window >= 0 && keep_first >= 0 && (chunk == 0 || window == 0) && (window > 0 || keep_first == 0),
+                  "attention_general: mask chunk %d, window %d, kept first tokens %d (a chunk or a window, not both; "
+                  "kept tokens only with a window)", chunk, window, keep_first);
     PagedView pv{page_table, table_width, page_size};
     dim3 grid(n, nh);
     if (dtype == CPMCU_F32)
         attention_general_kernel<float><<<grid, 64, 0, stream>>>((const float*)q, (float*)out, (const float*)kpool,
                                                                  (const float*)vpool, pv, positions, tok_slot, nh, nkv,
-                                                                 hdk, hdv, pool_hdk, pool_hdv, scale, chunk);
+                                                                 hdk, hdv, pool_hdk, pool_hdv, scale, chunk, window,
+                                                                 keep_first, sink);
     else if (dtype == CPMCU_BF16)
         attention_general_kernel<bf16_t><<<grid, 64, 0, stream>>>((const bf16_t*)q, (bf16_t*)out, (const bf16_t*)kpool,
                                                                   (const bf16_t*)vpool, pv, positions, tok_slot, nh,
-                                                                  nkv, hdk, hdv, pool_hdk, pool_hdv, scale, chunk);
+                                                                  nkv, hdk, hdv, pool_hdk, pool_hdv, scale, chunk, window,
+                                                                  keep_first, sink);
     else
         CPMCU_FAIL("attention_general: unknown dtype %d", dtype);
     CPMCU_LAUNCH_CHECK("attention_general");
@@ -195,7 +207,9 @@ extern "C" const char* cpmcu_attention_general(const void* q, void* out, int dty
 //   P^T = exp2(S^T c - m) in float per head, running maximum and sum
 //   O^T += V^T . P^T  A = V^T, 16 features x 32 keys a tile; the output of up to DTM tiles stays in registers
 // The mask is causal, and with chunk > 0 the keys before the start of the query's chunk are skipped (whole
-// 32-key chunks) or masked.  Output: out (bf16) when n_splits == 1, else unnormalised shares part_o
+// 32-key chunks) or masked; with window > 0 the keys more than window - 1 positions back are, except the first
+// keep_first keys of the sequence, whose 32-key chunks are visited before the window's.  With `sink` the
+// denominator gains exp(sink[head]) at the end (here, or in the merge kernel when the keys are split).  Output: out (bf16) when n_splits == 1, else unnormalised shares part_o
 // [token][head][split][hdv] and part_ml [token][head][split] = (max, sum) for the merge kernel below.
 // ===========================================================================
 typedef __bf16 gbf16x8_t __attribute__((ext_vector_type(8)));
@@ -210,8 +224,8 @@ __global__ __launch_bounds__(NW * TW * 64) void attention_general_mfma_kernel(
     const bf16_t* __restrict__ q, bf16_t* __restrict__ out, float* __restrict__ part_o, float2* __restrict__ part_ml,
     const bf16_t* __restrict__ kpool, const bf16_t* __restrict__ vtpool, PagedView pv,
     const int* __restrict__ positions, const int* __restrict__ tok_slot, int nh, int nkv, int hdk, int hdv,
-    int pool_hdk, int pool_hdv, float scale_log2e, int chunk, int n_splits, int n_tokens, const int* __restrict__ tiles,
-    int n_tiles, int tpt, int rpt) {
+    int pool_hdk, int pool_hdv, float scale_log2e, int chunk, int window, int keep_first, const float* __restrict__ sink,
+    int n_splits, int n_tokens, const int* __restrict__ tiles, int n_tiles, int tpt, int rpt) {
     extern __shared__ __align__(16) unsigned char smem[];
     static_assert(NW == 1 || TW == 1, "either the wavefronts of a workgroup share a token or each has its own");
     const int ksteps = (pool_hdk + 31) >> 5, dtn = pool_hdv >> 4;
@@ -245,10 +259,13 @@ __global__ __launch_bounds__(NW * TW * 64) void attention_general_mfma_kernel(
     }
     __syncthreads();
 
-    const int first_key = chunk > 0 ? pos - pos % chunk : 0;
-    const int first_min = chunk > 0 ? pos_min - pos_min % chunk : 0, first_max = chunk > 0 ? pos_max - pos_max % chunk : 0;
+    const int first_key = chunk > 0 ? pos - pos % chunk : (window > 0 ? max(pos - window + 1, 0) : 0);
+    const int first_min = chunk > 0 ? pos_min - pos_min % chunk : (window > 0 ? max(pos_min - window + 1, 0) : 0);
+    const int first_max = chunk > 0 ? pos_max - pos_max % chunk : (window > 0 ? max(pos_max - window + 1, 0) : 0);
     const int cfirst = first_min >> 5;
-    const int total_chunks = (pos_max >> 5) + 1 - cfirst;
+    // 32-key chunks of the kept first tokens that lie before the window's first chunk come first in the list
+    const int ckeep = min((keep_first + 31) >> 5, cfirst);
+    const int total_chunks = ckeep + (pos_max >> 5) + 1 - cfirst;
     const int per_split = (total_chunks + n_splits - 1) / n_splits;
     const int c0 = split * per_split, c1 = min(c0 + per_split, total_chunks);
 
@@ -266,7 +283,7 @@ __global__ __launch_bounds__(NW * TW * 64) void attention_general_mfma_kernel(
     float* sc_s = (float*)(smem + (long)ksteps * 64 * 16);        // VS: partial scores, behind the Q fragments
     int parity = 0;
     for (int c = VS ? c0 : c0 + wave; c < c1; c += VS ? 1 : NW) {
-        const int key0 = (cfirst + c) << 5;
+        const int key0 = (c < ckeep ? c : cfirst + (c - ckeep)) << 5;
         const long pchunk = paged_row(pv, slot, key0) >> 5;
         const bf16_t* kp = kpool + (pchunk * nkv + kvh) * kchunk + lane_off;
         const bf16_t* vp = vtpool + (pchunk * nkv + kvh) * vchunk + lane_off;
@@ -314,12 +331,12 @@ __global__ __launch_bounds__(NW * TW * 64) void attention_general_mfma_kernel(
             }
         }
         // lane (head n, g): st0[e] is key key0 + 8g + e, st1[e] is key key0 + 8g + 4 + e
-        if (key0 + 31 > pos_min || key0 < first_max) {
+        if (key0 + 31 > pos_min || (key0 < first_max && key0 + 31 >= keep_first)) {
 #pragma unroll
             for (int e = 0; e < 4; ++e) {
                 const int ka = key0 + 8 * g + e, kb = ka + 4;
-                if (ka > pos || ka < first_key) st0[e] = -INFINITY;
-                if (kb > pos || kb < first_key) st1[e] = -INFINITY;
+                if (ka > pos || (ka < first_key && ka >= keep_first)) st0[e] = -INFINITY;
+                if (kb > pos || (kb < first_key && kb >= keep_first)) st1[e] = -INFINITY;
             }
         }
         float mx = fmaxf(fmaxf(fmaxf(st0[0], st0[1]), fmaxf(st0[2], st0[3])),
@@ -393,6 +410,7 @@ __global__ __launch_bounds__(NW * TW * 64) void attention_general_mfma_kernel(
     if (!head_ok || !live) return;
     // lane (head n, g): acc[dt][i] is O[head][dt*16 + 4g + i]
     if (n_splits == 1) {
+        if (sink) l += exp2f(sink[head] * 1.4426950408889634f - m);
         const float inv = 1.0f / l;
         bf16_t* o = out + ((long)t * nh + head) * hdv;
 #pragma unroll
@@ -419,7 +437,8 @@ __global__ __launch_bounds__(NW * TW * 64) void attention_general_mfma_kernel(
 // out[token][head][:] = sum_s 2^(m_s - m) o_s / sum_s 2^(m_s - m) l_s over up to 64 shares (a share without keys
 // has l = 0): lane s holds share s's (max, sum), the common maximum and the denominator are wave reductions.
 __global__ void attention_general_merge_kernel(const float* __restrict__ part_o, const float2* __restrict__ part_ml,
-                                               bf16_t* __restrict__ out, int hdv, int n_splits) {
+                                               bf16_t* __restrict__ out, int hdv, int n_splits,
+                                               const float* __restrict__ sink, int nh) {
     const long row = blockIdx.x;
     const float2* ml = part_ml + row * n_splits;
     const float* po = part_o + row * n_splits * hdv;
@@ -429,7 +448,9 @@ __global__ void attention_general_merge_kernel(const float* __restrict__ part_o,
     const bool has = v.y > 0.f;
     const float m = wave_max(has ? v.x : -INFINITY);
     const float wv = has ? exp2f(v.x - m) : 0.f;
-    const float inv = 1.0f / wave_sum(wv * v.y);
+    // rows are (token, head): the sink of the row's head joins the denominator once
+    const float extra = sink ? exp2f(sink[row % nh] * 1.4426950408889634f - m) : 0.f;
+    const float inv = 1.0f / (wave_sum(wv * v.y) + extra);
     for (int d = threadIdx.x; d < hdv; d += blockDim.x) {
         float a = 0.f;
         int s = 0;
@@ -449,7 +470,8 @@ __global__ void attention_general_merge_kernel(const float* __restrict__ part_o,
 
 extern "C" const char* cpmcu_attention_general_mfma(const void* q, void* out, float* part_o, float* part_ml, int n,
                                                     int nh, int nkv, int hdk, int hdv, int pool_hdk, int pool_hdv,
-                                                    float scale, int chunk, const void* kpool, const void* vtpool,
+                                                    float scale, int chunk, int window, int keep_first,
+                                                    const float* sink, const void* kpool, const void* vtpool,
                                                     const int* page_table, int table_width, int page_size,
                                                     const int* positions, const int* tok_slot, int n_splits,
                                                     const int* tiles, int n_tiles, int tokens_per_tile,
@@ -462,7 +484,9 @@ extern "C" const char* cpmcu_attention_general_mfma(const void* q, void* out, fl
                   "attention_general_mfma: the cache holds heads in steps of 16 features and pages of a multiple of 32 tokens");
     CPMCU_REQUIRE(n_splits >= 1 && n_splits <= 64 && (n_splits == 1 || (part_o && part_ml)),
                   "attention_general_mfma: %d shares of the keys (1..64 are taken)", n_splits);
-    CPMCU_REQUIRE(chunk >= 0, "attention_general_mfma: mask chunk %d", chunk);
+    CPMCU_REQUIRE(chunk >= 0 && window >= 0 && keep_first >= 0 && (chunk == 0 || window == 0) && (window > 0 || keep_first == 0),
+                  "attention_general_mfma: mask chunk %d, window %d, kept first tokens %d (a chunk or a window, not both; "
+                  "kept tokens only with a window)", chunk, window, keep_first);
     const int G = nh / nkv, HT = (G + 15) / 16;
     CPMCU_REQUIRE((long)nkv * HT <= 65535, "attention_general_mfma: too many head tiles");
     PagedView pv{page_table, table_width, page_size};
@@ -491,7 +515,8 @@ extern "C" const char* cpmcu_attention_general_mfma(const void* q, void* out, fl
 #define LAUNCH(DTMv, NWv, TWv, VSv)                                                                              \
     attention_general_mfma_kernel<DTMv, NWv, TWv, VSv><<<grid, NWv * TWv * 64, lds, stream>>>(                   \
         (const bf16_t*)q, (bf16_t*)out, part_o, (float2*)part_ml, (const bf16_t*)kpool, (const bf16_t*)vtpool, pv, \
-        positions, tok_slot, nh, nkv, hdk, hdv, pool_hdk, pool_hdv, sl, chunk, n_splits, n, tiles, n_tiles, tpt, rpt)
+        positions, tok_slot, nh, nkv, hdk, hdv, pool_hdk, pool_hdv, sl, chunk, window, keep_first, sink, n_splits, n,    \
+        tiles, n_tiles, tpt, rpt)
     if (vs) {
         if (dtm == 4) LAUNCH(4, 4, 1, true);
         else LAUNCH(8, 4, 1, true);
@@ -510,7 +535,7 @@ extern "C" const char* cpmcu_attention_general_mfma(const void* q, void* out, fl
     if (n_splits > 1) {
         const unsigned rows = (unsigned)((long)n * nh);
         attention_general_merge_kernel<<<rows, hdv > 128 ? 256 : (hdv > 64 ? 128 : 64), 0, stream>>>(
-            part_o, (const float2*)part_ml, (bf16_t*)out, hdv, n_splits);
+            part_o, (const float2*)part_ml, (bf16_t*)out, hdv, n_splits, sink, nh);
         CPMCU_LAUNCH_CHECK("attention_general_merge");
     }
     return nullptr;
@@ -594,6 +619,91 @@ extern "C" const char* cpmcu_qkv_rotate_store(const void* qkv, long ld, int dtyp
     else
         CPMCU_FAIL("qkv_rotate_store: unknown dtype %d", dtype);
     CPMCU_LAUNCH_CHECK("qkv_rotate_store");
+    return nullptr;
+}
+
+// The same for designs that put more between projection and rotation, in one launch, grid (tokens, nh + nkv or
+// nh + 2 nkv), a wavefront a (token, head), everything in float:
+//   * `bias` (float, as wide as the projection's row) is added to the projection;
+//   * q heads and k heads are divided by their root mean square (eps inside the root) and multiplied by a weight
+//     of dk numbers shared by the heads (q_norm_w, k_norm_w; either may be absent), before the rotation;
+//   * with values_from_keys the row holds no v: the value pages receive k as projected (with its bias, before norm
+//     and rotation), so dv == dk.
+template <typename T>
+__global__ __launch_bounds__(64) void qkv_norm_rotate_store_kernel(
+    const T* __restrict__ qkv, long ld, const float* __restrict__ bias, T* __restrict__ q_out, int nh, int nkv, int dk,
+    int dv, int rot_dims, const float* __restrict__ q_norm_w, const float* __restrict__ k_norm_w, float eps,
+    int values_from_keys, const int* __restrict__ positions, const int* __restrict__ tok_slot,
+    const float* __restrict__ inv_freq, float mag, T* __restrict__ kpool, T* __restrict__ vpool, PagedView pv,
+    int pool_hdk, int pool_hdv) {
+    __shared__ float hs[AG_MAX_HD];
+    const long t = blockIdx.x;
+    const int y = blockIdx.y, lane = threadIdx.x;
+    const int pos = positions[t];
+    const bool is_q = y < nh, is_k = !is_q && y < nh + nkv;
+    const int h = is_q ? y : (is_k ? y - nh : y - nh - nkv);
+    const int width = (is_q || is_k) ? dk : dv;
+    const long col = is_q ? (long)h * dk : (is_k ? (long)(nh + h) * dk : (long)(nh + nkv) * dk + (long)h * dv);
+    const T* src = qkv + t * ld + col;
+    const long prow = is_q ? 0 : paged_row(pv, tok_slot[t], pos);
+    if (!is_q && !is_k) {               // a value head of its own: copied as it is
+        T* vd = vpool + value_index(prow, h, nkv, pool_hdv);
+        for (int i = lane; i < dv; i += 64) vd[value_d_offset(i)] = from_f32<T>(to_f32(src[i]) + (bias ? bias[col + i] : 0.f));
+        return;
+    }
+    float ss = 0.f;
+    for (int i = lane; i < width; i += 64) {
+        const float v = to_f32(src[i]) + (bias ? bias[col + i] : 0.f);
+        hs[i] = v;
+        ss += v * v;
+    }
+    if (is_k && values_from_keys) {
+        T* vd = vpool + value_index(prow, h, nkv, pool_hdv);
+        for (int i = lane; i < width; i += 64) vd[value_d_offset(i)] = from_f32<T>(hs[i]);
+    }
+    const float* nw = is_q ? q_norm_w : k_norm_w;
+    if (nw) {
+        const float r = 1.0f / sqrtf(wave_sum(ss) / (float)width + eps);
+        for (int i = lane; i < width; i += 64) hs[i] = hs[i] * r * nw[i];
+    }
+    __syncthreads();
+    if (is_q) rotate_run(hs, q_out + (t * nh + h) * dk, dk, rot_dims, pos, inv_freq, mag, DST_ROWS, 0, lane, 64);
+    else rotate_run(hs, kpool + key_index(prow, h, nkv, pool_hdk), dk, rot_dims, pos, inv_freq, mag, DST_KEYS, 0, lane, 64);
+}
+
+extern "C" const char* cpmcu_qkv_norm_rotate_store(const void* qkv, long ld, int dtype, const float* bias, void* q_out,
+                                                   int n, int nh, int nkv, int dk, int dv, int rot_dims,
+                                                   const float* q_norm_w, const float* k_norm_w, float eps,
+                                                   int values_from_keys, const int* positions, const int* tok_slot,
+                                                   const float* inv_freq, float mag, void* kpool, void* vpool,
+                                                   const int* page_table, int table_width, int page_size, int pool_hdk,
+                                                   int pool_hdv, int write_kv, hipStream_t stream) {
+    CPMCU_REQUIRE(n > 0 && nh > 0 && nkv > 0 && dk > 0 && dv > 0, "qkv_norm_rotate_store: empty shape");
+    CPMCU_REQUIRE(dk <= AG_MAX_HD && dv <= AG_MAX_HD, "qkv_norm_rotate_store: key size %d / value size %d (up to %d are taken)",
+                  dk, dv, AG_MAX_HD);
+    CPMCU_REQUIRE(rot_dims >= 0 && rot_dims % 2 == 0 && rot_dims <= dk && (rot_dims == 0 || inv_freq),
+                  "qkv_norm_rotate_store: %d rotated features of %d", rot_dims, dk);
+    CPMCU_REQUIRE(!values_from_keys || dv == dk, "qkv_norm_rotate_store: values that are the keys have the keys' size (%d, %d)", dv, dk);
+    const long row = (long)nh * dk + (write_kv ? (long)nkv * dk + (values_from_keys ? 0 : (long)nkv * dv) : 0);
+    CPMCU_REQUIRE(ld >= row, "qkv_norm_rotate_store: rows of %ld too short", ld);
+    CPMCU_REQUIRE(!write_kv || (kpool && vpool && page_table && page_size % 32 == 0 && pool_hdk % 16 == 0 &&
+                                pool_hdv % 16 == 0 && pool_hdk >= dk && pool_hdv >= dv),
+                  "qkv_norm_rotate_store: the cache takes pages of a multiple of 32 tokens and head sizes in steps of 16");
+    const int heads = nh + (write_kv ? (values_from_keys ? nkv : 2 * nkv) : 0);
+    CPMCU_REQUIRE(heads <= 65535, "qkv_norm_rotate_store: %d heads exceed the launch grid", heads);
+    PagedView pv{page_table, table_width, page_size};
+    dim3 grid(n, heads);
+    if (dtype == CPMCU_F32)
+        qkv_norm_rotate_store_kernel<float><<<grid, 64, 0, stream>>>(
+            (const float*)qkv, ld, bias, (float*)q_out, nh, nkv, dk, dv, rot_dims, q_norm_w, k_norm_w, eps, values_from_keys,
+            positions, tok_slot, inv_freq, mag, (float*)kpool, (float*)vpool, pv, pool_hdk, pool_hdv);
+    else if (dtype == CPMCU_BF16)
+        qkv_norm_rotate_store_kernel<bf16_t><<<grid, 64, 0, stream>>>(
+            (const bf16_t*)qkv, ld, bias, (bf16_t*)q_out, nh, nkv, dk, dv, rot_dims, q_norm_w, k_norm_w, eps,
+            values_from_keys, positions, tok_slot, inv_freq, mag, (bf16_t*)kpool, (bf16_t*)vpool, pv, pool_hdk, pool_hdv);
+    else
+        CPMCU_FAIL("qkv_norm_rotate_store: unknown dtype %d", dtype);
+    CPMCU_LAUNCH_CHECK("qkv_norm_rotate_store");
     return nullptr;
 }
 

@@ -30,8 +30,10 @@ MODULES: Dict[str, List[str]] = {
     "attention": ["attention.hip"],
     "sparse": ["sparse.hip"],
     "qkv": ["qkv_rope.hip", "strip.hip"],
-    "norms": ["norms.hip"],
+    "norms": ["norms.hip", "residual.hip"],
     "ssm": ["ssm.hip"],
+    "mlstm": ["mlstm.hip"],
+    "moe": ["moe.hip"],
     "attention_general": ["attention_general.hip"],
 }
 HEADERS = ["common.h"]

@@ -1,0 +1,262 @@
+// A feed-forward of routed experts, for steps of any number of tokens and both element types:
+//
+//  * moe_route_kernel: router logits z = Wr h in float (Wr float [E, H]), s = softmax(z); choice scores c = s +
+//    correction; the experts form `n_groups` equal groups of neighbours, a group's score is its largest c, and only
+//    experts of the `keep_groups` best groups may be chosen (n_groups = 1: any); the `top` largest c are chosen
+//    (ties: the lower index), their weights are s / (sum of the chosen s + 1e-20).  With w_sg (float [H]) it also
+//    gives sigmoid(w_sg . h), the gate of an expert that every token uses.
+//  * moe_gated_kernel: act[t, k, :] = silu(Wg_e h_t) * (Wu_e h_t) for the k-th chosen expert e of token t; the
+//    experts' gate and up rows are stacked: wgu [E, 2F, H], gate rows first.
+//  * moe_down_kernel: out[t] = sum_k w[t, k] Wd_e act[t, k] (+ sg[t] * shared[t]); wd [E, H, F]; float out.
+//
+// A wavefront owns output rows and its lanes stride over the input features (16-byte loads when the rows are
+// aligned), so an expert's weights stream once for every token that chose it: the form for steps of few tokens.
+#include "common.h"
+
+#define MOE_MAX_EXPERTS 1024
+
+template <typename T> struct Vec8;
+template <> struct Vec8<bf16_t> { typedef uint4 type; };
+template <> struct Vec8<float> { struct type { float4 a, b; }; };
+
+template <typename T>
+__device__ inline void load8(const T* p, float* v);
+template <>
+__device__ inline void load8<bf16_t>(const bf16_t* p, float* v) {
+    const uint4 u = *(const uint4*)p;
+    const uint32_t w[4] = {u.x, u.y, u.z, u.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        v[2 * i] = __uint_as_float(w[i] << 16);
+        v[2 * i + 1] = __uint_as_float(w[i] & 0xffff0000u);
+    }
+}
+template <>
+__device__ inline void load8<float>(const float* p, float* v) {
+    const float4 a = *(const float4*)p, b = *(const float4*)(p + 4);
+    v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w;
+    v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+}
+
+// the lane's share of dot(a[0:K], b[0:K]); `vec`: both rows are 16-byte aligned (32 for float) and K % 8 == 0
+template <typename TA, typename TB>
+__device__ inline float lane_dot(const TA* __restrict__ a, const TB* __restrict__ b, int K, int lane, bool vec) {
+    float s = 0.f;
+    if (vec) {
+        for (int c = lane * 8; c < K; c += 64 * 8) {
+            float x[8], y[8];
+            load8<TA>(a + c, x);
+            load8<TB>(b + c, y);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) s += x[i] * y[i];
+        }
+    } else {
+        for (int c = lane; c < K; c += 64) s += to_f32(a[c]) * to_f32(b[c]);
+    }
+    return s;
+}
+
+__device__ inline float wave_min_f(float v) { return -wave_max(-v); }
+
+// grid (tokens), 256 threads
+template <typename T>
+__global__ __launch_bounds__(256) void moe_route_kernel(const T* __restrict__ h, long ldh, const float* __restrict__ wr,
+                                                        const float* __restrict__ correction,
+                                                        const float* __restrict__ w_sg, int H, int E, int n_groups,
+                                                        int keep_groups, int top, int* __restrict__ idx_out,
+                                                        float* __restrict__ w_out, float* __restrict__ sg_out) {
+    __shared__ float z[MOE_MAX_EXPERTS];      // logits, then softmax scores
+    __shared__ float c[MOE_MAX_EXPERTS];      // choice scores; -inf once an expert is chosen or shut out
+    __shared__ float gs[MOE_MAX_EXPERTS];     // group scores
+    const long t = blockIdx.x;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const T* hr = h + t * ldh;
+    const bool vec = (H % 8 == 0) && (ldh % 8 == 0) && ((uintptr_t)h % 32 == 0) && ((uintptr_t)wr % 32 == 0);
+    for (int e = wave; e < E + (w_sg ? 1 : 0); e += 4) {
+        const float* row = e < E ? wr + (long)e * H : w_sg;
+        const bool v = vec && (e < E || (uintptr_t)w_sg % 32 == 0);
+        const float s = wave_sum(lane_dot<T, float>(hr, row, H, lane, v));
+        if (lane == 0) {
+            if (e < E) z[e] = s;
+            else sg_out[t] = 1.0f / (1.0f + expf(-s));
+        }
+    }
+    __syncthreads();
+    if (wave != 0) return;
+    float mx = -INFINITY;
+    for (int e = lane; e < E; e += 64) mx = fmaxf(mx, z[e]);
+    mx = wave_max(mx);
+    float sum = 0.f;
+    for (int e = lane; e < E; e += 64) {
+        const float p = expf(z[e] - mx);
+        z[e] = p;
+        sum += p;
+    }
+    sum = wave_sum(sum);
+    const float inv = 1.0f / sum;
+    for (int e = lane; e < E; e += 64) {
+        z[e] *= inv;
+        c[e] = z[e] + (correction ? correction[e] : 0.f);
+    }
+    __builtin_amdgcn_wave_barrier();
+    if (n_groups > 1) {
+        const int per = E / n_groups;
+        for (int g = lane; g < n_groups; g += 64) {
+            float b = -INFINITY;
+            for (int i = 0; i < per; ++i) b = fmaxf(b, c[g * per + i]);
+            gs[g] = b;
+        }
+        __builtin_amdgcn_wave_barrier();
+        // the best groups, one a turn, are marked with +inf; afterwards every other group's experts are shut out
+        for (int r = 0; r < keep_groups; ++r) {
+            float b = -INFINITY;
+            for (int g = lane; g < n_groups; g += 64)
+                if (gs[g] != INFINITY) b = fmaxf(b, gs[g]);
+            b = wave_max(b);
+            float first = 3.0e38f;
+            for (int g = lane; g < n_groups; g += 64)
+                if (gs[g] != INFINITY && gs[g] == b) first = fminf(first, (float)g);
+            const int win = (int)wave_min_f(first);
+            if (lane == 0) gs[win] = INFINITY;
+            __builtin_amdgcn_wave_barrier();
+        }
+        for (int e = lane; e < E; e += 64)
+            if (gs[e / per] != INFINITY) c[e] = -INFINITY;
+        __builtin_amdgcn_wave_barrier();
+    }
+    float chosen_sum = 0.f;
+    for (int r = 0; r < top; ++r) {
+        float b = -INFINITY;
+        for (int e = lane; e < E; e += 64) b = fmaxf(b, c[e]);
+        b = wave_max(b);
+        float first = 3.0e38f;
+        for (int e = lane; e < E; e += 64)
+            if (c[e] == b) first = fminf(first, (float)e);
+        const int win = (int)wave_min_f(first);
+        chosen_sum += z[win];
+        if (lane == 0) {
+            idx_out[t * top + r] = win;
+            w_out[t * top + r] = z[win];
+            c[win] = -INFINITY;
+        }
+        __builtin_amdgcn_wave_barrier();
+    }
+    const float norm = 1.0f / (chosen_sum + 1e-20f);
+    for (int r = lane; r < top; r += 64) w_out[t * top + r] *= norm;
+}
+
+extern "C" const char* cpmcu_moe_route(const void* h, long ldh, int dtype, const float* wr, const float* correction,
+                                       const float* w_sg, int n, int H, int E, int n_groups, int keep_groups, int top,
+                                       int* idx_out, float* w_out, float* sg_out, hipStream_t stream) {
+    CPMCU_REQUIRE(n > 0 && H > 0 && E > 0, "moe_route: empty shape");
+    CPMCU_REQUIRE(E <= MOE_MAX_EXPERTS, "moe_route: %d experts (up to %d are taken)", E, MOE_MAX_EXPERTS);
+    CPMCU_REQUIRE(n_groups >= 1 && E % n_groups == 0 && keep_groups >= 1 && keep_groups <= n_groups,
+                  "moe_route: %d experts in %d groups of which %d may be chosen from", E, n_groups, keep_groups);
+    CPMCU_REQUIRE(top >= 1 && top <= keep_groups * (E / n_groups), "moe_route: %d experts a token of %d that may be chosen",
+                  top, keep_groups * (E / n_groups));
+    CPMCU_REQUIRE(!w_sg || sg_out, "moe_route: a place for the shared gate is missing");
+    if (dtype == CPMCU_F32)
+        moe_route_kernel<float><<<n, 256, 0, stream>>>((const float*)h, ldh, wr, correction, w_sg, H, E, n_groups,
+                                                       keep_groups, top, idx_out, w_out, sg_out);
+    else if (dtype == CPMCU_BF16)
+        moe_route_kernel<bf16_t><<<n, 256, 0, stream>>>((const bf16_t*)h, ldh, wr, correction, w_sg, H, E, n_groups,
+                                                        keep_groups, top, idx_out, w_out, sg_out);
+    else
+        CPMCU_FAIL("moe_route: unknown dtype %d", dtype);
+    CPMCU_LAUNCH_CHECK("moe_route");
+    return nullptr;
+}
+
+#define MOE_ROWS 4       // output rows a wavefront
+
+// grid (tokens * top, ceil(F / 16)), 256 threads: wavefront w takes rows [16 y + 4 w, +4) of the expert's F
+template <typename T>
+__global__ __launch_bounds__(256) void moe_gated_kernel(const T* __restrict__ h, long ldh, const T* __restrict__ wgu,
+                                                        const int* __restrict__ idx, T* __restrict__ act, int H, int F,
+                                                        int top) {
+    const long pair = blockIdx.x;
+    const long t = pair / top;
+    const int e = idx[pair];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const T* hr = h + t * ldh;
+    const T* wg = wgu + (long)e * 2 * F * H;
+    const bool vec = (H % 8 == 0) && (ldh % 8 == 0) && ((uintptr_t)h % 32 == 0) && ((uintptr_t)wgu % 32 == 0);
+    const int j0 = blockIdx.y * 4 * MOE_ROWS + wave * MOE_ROWS;
+#pragma unroll
+    for (int r = 0; r < MOE_ROWS; ++r) {
+        const int j = j0 + r;
+        if (j >= F) break;
+        const float g = wave_sum(lane_dot<T, T>(wg + (long)j * H, hr, H, lane, vec));
+        const float u = wave_sum(lane_dot<T, T>(wg + (long)(F + j) * H, hr, H, lane, vec));
+        if (lane == 0) act[pair * F + j] = from_f32<T>(g / (1.0f + expf(-g)) * u);
+    }
+}
+
+extern "C" const char* cpmcu_moe_gated(const void* h, long ldh, int dtype, const void* wgu, const int* idx, void* act,
+                                       int n, int H, int F, int top, hipStream_t stream) {
+    CPMCU_REQUIRE(n > 0 && H > 0 && F > 0 && top > 0, "moe_gated: empty shape");
+    const int fy = (F + 4 * MOE_ROWS - 1) / (4 * MOE_ROWS);
+    CPMCU_REQUIRE(fy <= 65535, "moe_gated: %d rows an expert exceed the launch grid", F);
+    dim3 grid((unsigned)((long)n * top), fy);
+    if (dtype == CPMCU_F32)
+        moe_gated_kernel<float><<<grid, 256, 0, stream>>>((const float*)h, ldh, (const float*)wgu, idx, (float*)act, H, F, top);
+    else if (dtype == CPMCU_BF16)
+        moe_gated_kernel<bf16_t><<<grid, 256, 0, stream>>>((const bf16_t*)h, ldh, (const bf16_t*)wgu, idx, (bf16_t*)act, H, F, top);
+    else
+        CPMCU_FAIL("moe_gated: unknown dtype %d", dtype);
+    CPMCU_LAUNCH_CHECK("moe_gated");
+    return nullptr;
+}
+
+// grid (tokens, ceil(H / 16)), 256 threads.  shared: the every-token expert's output [n, H] (or float partial
+// sums [parts][n][H]), multiplied by sg[t]; may be absent.
+template <typename T, typename ST>
+__global__ __launch_bounds__(256) void moe_down_kernel(const T* __restrict__ act, const T* __restrict__ wd,
+                                                       const int* __restrict__ idx, const float* __restrict__ w,
+                                                       const ST* __restrict__ shared, int shared_parts,
+                                                       long shared_stride, const float* __restrict__ sg,
+                                                       float* __restrict__ out, int H, int F, int top) {
+    const long t = blockIdx.x;
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const bool vec = (F % 8 == 0) && ((uintptr_t)act % 32 == 0) && ((uintptr_t)wd % 32 == 0);
+    const int c0 = blockIdx.y * 4 * MOE_ROWS + wave * MOE_ROWS;
+#pragma unroll
+    for (int r = 0; r < MOE_ROWS; ++r) {
+        const int c = c0 + r;
+        if (c >= H) break;
+        float s = 0.f;
+        for (int k = 0; k < top; ++k) {
+            const int e = idx[t * top + k];
+            s += w[t * top + k] * lane_dot<T, T>(wd + ((long)e * H + c) * F, act + (t * top + k) * F, F, lane, vec);
+        }
+        s = wave_sum(s);
+        if (lane == 0) {
+            if (shared) {
+                float v = 0.f;
+                for (int p = 0; p < shared_parts; ++p) v += to_f32(shared[(long)p * shared_stride + t * H + c]);
+                s += (sg ? sg[t] : 1.0f) * v;
+            }
+            out[t * H + c] = s;
+        }
+    }
+}
+
+extern "C" const char* cpmcu_moe_down(const void* act, int dtype, const void* wd, const int* idx, const float* w,
+                                      const void* shared, int shared_dtype, int shared_parts, long shared_stride,
+                                      const float* sg, float* out, int n, int H, int F, int top, hipStream_t stream) {
+    CPMCU_REQUIRE(n > 0 && H > 0 && F > 0 && top > 0, "moe_down: empty shape");
+    const int hy = (H + 4 * MOE_ROWS - 1) / (4 * MOE_ROWS);
+    CPMCU_REQUIRE(hy <= 65535, "moe_down: a width of %d exceeds the launch grid", H);
+    dim3 grid(n, hy);
+#define LAUNCH(Tv, STv)                                                                                            \
+    moe_down_kernel<Tv, STv><<<grid, 256, 0, stream>>>((const Tv*)act, (const Tv*)wd, idx, w, (const STv*)shared,   \
+                                                       shared_parts, shared_stride, sg, out, H, F, top)
+    const int sd = shared ? shared_dtype : CPMCU_F32;
+    if (dtype == CPMCU_F32 && sd == CPMCU_F32) LAUNCH(float, float);
+    else if (dtype == CPMCU_BF16 && sd == CPMCU_F32) LAUNCH(bf16_t, float);
+    else if (dtype == CPMCU_BF16 && sd == CPMCU_BF16) LAUNCH(bf16_t, bf16_t);
+    else CPMCU_FAIL("moe_down: unsupported dtypes act=%d shared=%d", dtype, sd);
+#undef LAUNCH
+    CPMCU_LAUNCH_CHECK("moe_down");
+    return nullptr;
+}

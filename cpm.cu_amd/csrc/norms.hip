@@ -1,7 +1,8 @@
 // Norms beyond the residual RMSNorm of elementwise.hip, all with float statistics:
 //
 //  * rms_norm_groups_kernel: RMS norm of a row cut into equal groups, each by its own root mean square,
-//    optionally after a SiLU gate (y <- y * silu(z), the gate before the norm).  Rows may be slices of wider
+//    optionally after a SiLU gate (y <- y * silu(z), the gate before the norm) or followed by a sigmoid gate
+//    (out <- norm(y) * w * sigmoid(z), the gate after the norm).  Rows may be slices of wider
 //    rows (leading dimensions), so the first columns of a projection are normed where they lie.
 //  * branch_norm_add_norm_kernel: a branch that has a norm of its own before it joins the residual
 //    (x += rmsnorm(b) * wb), then the norm of the next sub-layer on the sum (out = rmsnorm(x) * w): the
@@ -21,21 +22,23 @@ __device__ inline float sum_slices(const T* p, int nparts, long stride) {
 
 __device__ inline float silu_f(float z) { return z / (1.0f + expf(-z)); }
 
-// grid (rows, groups); out[r, g*W + c] = v * rsqrt(mean_g(v^2) + eps) * weight[g*W + c], v = x * silu(z) if z
+// grid (rows, groups); out[r, g*W + c] = v * rsqrt(mean_g(v^2) + eps) * weight[g*W + c], v = x * silu(z) if z and
+// gate_after == 0; with gate_after the statistics are those of x alone and the result is multiplied by sigmoid(z)
 template <typename XT, typename ZT, typename OT>
 __global__ __launch_bounds__(256) void rms_norm_groups_kernel(const XT* __restrict__ x, long ldx,
                                                               const ZT* __restrict__ z, long ldz,
                                                               const float* __restrict__ weight, OT* __restrict__ out,
-                                                              long ldo, int W, float eps) {
+                                                              long ldo, int W, float eps, int gate_after) {
     __shared__ float red[17];
     const long r = blockIdx.x;
     const int g = blockIdx.y;
     const XT* xr = x + r * ldx + (long)g * W;
     const ZT* zr = z ? z + r * ldz + (long)g * W : nullptr;
+    const bool before = zr && !gate_after;
     float ss = 0.f;
     for (int c = threadIdx.x; c < W; c += blockDim.x) {
         float v = to_f32(xr[c]);
-        if (zr) v *= silu_f(to_f32(zr[c]));
+        if (before) v *= silu_f(to_f32(zr[c]));
         ss += v * v;
     }
     ss = block_sum(ss, red);
@@ -43,16 +46,17 @@ __global__ __launch_bounds__(256) void rms_norm_groups_kernel(const XT* __restri
     OT* orow = out + r * ldo + (long)g * W;
     for (int c = threadIdx.x; c < W; c += blockDim.x) {
         float v = to_f32(xr[c]);
-        if (zr) v *= silu_f(to_f32(zr[c]));
+        if (before) v *= silu_f(to_f32(zr[c]));
         v *= rs;
         if (weight) v *= weight[(long)g * W + c];
+        if (zr && gate_after) v *= 1.0f / (1.0f + expf(-to_f32(zr[c])));
         orow[c] = from_f32<OT>(v);
     }
 }
 
 extern "C" const char* cpmcu_rms_norm_groups(const void* x, long ldx, int x_dtype, const void* z, long ldz, int z_dtype,
                                              const float* weight, void* out, long ldo, int out_dtype, int n, int groups,
-                                             int W, float eps, hipStream_t stream) {
+                                             int W, float eps, int gate_after, hipStream_t stream) {
     CPMCU_REQUIRE(n > 0 && groups > 0 && W > 0, "rms_norm_groups: empty shape rows=%d groups=%d width=%d", n, groups, W);
     CPMCU_REQUIRE(groups <= 65535, "rms_norm_groups: %d groups exceed the launch grid", groups);
     CPMCU_REQUIRE(ldx >= (long)groups * W && ldo >= (long)groups * W && (!z || ldz >= (long)groups * W),
@@ -61,7 +65,7 @@ extern "C" const char* cpmcu_rms_norm_groups(const void* x, long ldx, int x_dtyp
     const int block = W >= 256 ? 256 : 64;
 #define LAUNCH(XT, ZT, OT)                                                                                     \
     rms_norm_groups_kernel<XT, ZT, OT><<<grid, block, 0, stream>>>((const XT*)x, ldx, (const ZT*)z, ldz, weight, \
-                                                                   (OT*)out, ldo, W, eps)
+                                                                   (OT*)out, ldo, W, eps, gate_after)
     const int zd = z ? z_dtype : x_dtype;
     if (x_dtype == CPMCU_F32 && zd == CPMCU_F32 && out_dtype == CPMCU_F32) LAUNCH(float, float, float);
     else if (x_dtype == CPMCU_F32 && zd == CPMCU_F32 && out_dtype == CPMCU_BF16) LAUNCH(float, float, bf16_t);

@@ -1,0 +1,83 @@
+// What joins sub-layers' results before they enter the residual stream:
+//
+//  * gated_branches_kernel: out = sigmoid(g1 + b1) * (A + a_bias) + sigmoid(g2 + b2) * F, element by element in
+//    float: two sub-layers that read the same normed rows (a parallel layer), each multiplied by a gate of its own
+//    that is a projection of those rows; [g1 | g2] are the columns of one product, [b1 | b2] its bias.  A and F
+//    may come as float partial sums [parts][n][H] of a split product; F (and its gate) may be absent.
+//  * bias_sum_kernel: out = sum of the parts + bias, for a consumer that knows nothing of biases.
+#include "common.h"
+
+template <typename GT, typename AT, typename FT>
+__global__ __launch_bounds__(256) void gated_branches_kernel(const GT* __restrict__ g, long ldg,
+                                                             const float* __restrict__ g_bias,
+                                                             const AT* __restrict__ a, int a_parts, long a_stride,
+                                                             const float* __restrict__ a_bias,
+                                                             const FT* __restrict__ f, int f_parts, long f_stride,
+                                                             const float* __restrict__ f_bias,
+                                                             float* __restrict__ out, long total, int H) {
+    for (long i = (long)blockIdx.x * 256 + threadIdx.x; i < total; i += (long)gridDim.x * 256) {
+        const long t = i / H;
+        const int c = (int)(i - t * H);
+        float av = a_bias ? a_bias[c] : 0.f;
+        for (int p = 0; p < a_parts; ++p) av += to_f32(a[(long)p * a_stride + i]);
+        const float g1 = to_f32(g[t * ldg + c]) + (g_bias ? g_bias[c] : 0.f);
+        float v = av / (1.0f + expf(-g1));
+        if (f) {
+            float fv = f_bias ? f_bias[c] : 0.f;
+            for (int p = 0; p < f_parts; ++p) fv += to_f32(f[(long)p * f_stride + i]);
+            const float g2 = to_f32(g[t * ldg + H + c]) + (g_bias ? g_bias[H + c] : 0.f);
+            v += fv / (1.0f + expf(-g2));
+        }
+        out[i] = v;
+    }
+}
+
+extern "C" const char* cpmcu_gated_branches(const void* g, long ldg, int g_dtype, const float* g_bias, const void* a,
+                                            int a_dtype, int a_parts, long a_stride, const float* a_bias, const void* f,
+                                            int f_dtype, int f_parts, long f_stride, const float* f_bias, float* out,
+                                            int n, int H, hipStream_t stream) {
+    CPMCU_REQUIRE(n > 0 && H > 0 && a && a_parts >= 1, "gated_branches: empty shape");
+    CPMCU_REQUIRE(ldg >= (f ? 2L : 1L) * H, "gated_branches: gate rows of %ld for %d columns", ldg, H);
+    const long total = (long)n * H;
+    const int blocks = (int)((total + 255) / 256 < 4096 ? (total + 255) / 256 : 4096);
+    const int fd = f ? f_dtype : a_dtype;
+#define LAUNCH(GT, AT, FT)                                                                                         \
+    gated_branches_kernel<GT, AT, FT><<<blocks, 256, 0, stream>>>((const GT*)g, ldg, g_bias, (const AT*)a, a_parts,  \
+                                                                  a_stride, a_bias, (const FT*)f, f_parts, f_stride, \
+                                                                  f_bias, out, total, H)
+    if (g_dtype == CPMCU_F32 && a_dtype == CPMCU_F32 && fd == CPMCU_F32) LAUNCH(float, float, float);
+    else if (g_dtype == CPMCU_BF16 && a_dtype == CPMCU_F32 && fd == CPMCU_F32) LAUNCH(bf16_t, float, float);
+    else if (g_dtype == CPMCU_BF16 && a_dtype == CPMCU_BF16 && fd == CPMCU_F32) LAUNCH(bf16_t, bf16_t, float);
+    else if (g_dtype == CPMCU_BF16 && a_dtype == CPMCU_F32 && fd == CPMCU_BF16) LAUNCH(bf16_t, float, bf16_t);
+    else if (g_dtype == CPMCU_BF16 && a_dtype == CPMCU_BF16 && fd == CPMCU_BF16) LAUNCH(bf16_t, bf16_t, bf16_t);
+    else if (g_dtype == CPMCU_F32 && a_dtype == CPMCU_BF16 && fd == CPMCU_BF16) LAUNCH(float, bf16_t, bf16_t);
+    else if (g_dtype == CPMCU_F32 && a_dtype == CPMCU_F32 && fd == CPMCU_BF16) LAUNCH(float, float, bf16_t);
+    else if (g_dtype == CPMCU_F32 && a_dtype == CPMCU_BF16 && fd == CPMCU_F32) LAUNCH(float, bf16_t, float);
+    else CPMCU_FAIL("gated_branches: unsupported dtypes gate=%d a=%d f=%d", g_dtype, a_dtype, fd);
+#undef LAUNCH
+    CPMCU_LAUNCH_CHECK("gated_branches");
+    return nullptr;
+}
+
+template <typename AT>
+__global__ __launch_bounds__(256) void bias_sum_kernel(const AT* __restrict__ a, int parts, long stride,
+                                                       const float* __restrict__ bias, float* __restrict__ out,
+                                                       long total, int H) {
+    for (long i = (long)blockIdx.x * 256 + threadIdx.x; i < total; i += (long)gridDim.x * 256) {
+        float v = bias[i % H];
+        for (int p = 0; p < parts; ++p) v += to_f32(a[(long)p * stride + i]);
+        out[i] = v;
+    }
+}
+
+extern "C" const char* cpmcu_bias_sum(const void* a, int dtype, int parts, long stride, const float* bias, float* out,
+                                      int n, int H, hipStream_t stream) {
+    CPMCU_REQUIRE(n > 0 && H > 0 && parts >= 1 && bias, "bias_sum: empty shape");
+    const long total = (long)n * H;
+    const int blocks = (int)((total + 255) / 256 < 4096 ? (total + 255) / 256 : 4096);
+    if (dtype == CPMCU_F32) bias_sum_kernel<float><<<blocks, 256, 0, stream>>>((const float*)a, parts, stride, bias, out, total, H);
+    else if (dtype == CPMCU_BF16) bias_sum_kernel<bf16_t><<<blocks, 256, 0, stream>>>((const bf16_t*)a, parts, stride, bias, out, total, H);
+    else CPMCU_FAIL("bias_sum: unknown dtype %d", dtype);
+    CPMCU_LAUNCH_CHECK("bias_sum");
+    return nullptr;
+}

@@ -457,10 +457,11 @@ def _ld(t: torch.Tensor, name: str) -> int:
 
 
 def rms_norm_groups(x: torch.Tensor, weight: Optional[torch.Tensor], eps: float, out: torch.Tensor, groups: int = 1,
-                    gate: Optional[torch.Tensor] = None):
+                    gate: Optional[torch.Tensor] = None, gate_after: bool = False):
     """out[r] = v / sqrt(mean(v^2) + eps) * weight, group by group (``groups`` equal parts of a row, each by its
-    own root mean square), v = x * silu(gate) when a gate is given (the gate comes before the norm).  x, gate
-    and out may be column slices of wider tensors; statistics in float."""
+    own root mean square), v = x * silu(gate) when a gate is given (the gate comes before the norm); with
+    ``gate_after`` v = x and the result is multiplied by sigmoid(gate) instead.  x, gate and out may be column
+    slices of wider tensors; statistics in float."""
     ldx, ldo = _ld(x, "norm x"), _ld(out, "norm out")
     n, width = x.shape
     if groups <= 0 or width % groups:
@@ -477,7 +478,8 @@ def rms_norm_groups(x: torch.Tensor, weight: Optional[torch.Tensor], eps: float,
     _check(_fn("norms", "cpmcu_rms_norm_groups")(_p(x), c_long(ldx), c_int(_code(x)), _p(gate), c_long(ldz),
                                                  c_int(_code(gate) if gate is not None else 0), _p(weight), _p(out),
                                                  c_long(ldo), c_int(_code(out)), c_int(n), c_int(groups),
-                                                 c_int(width // groups), c_float(eps), _stream()))
+                                                 c_int(width // groups), c_float(eps), c_int(1 if gate_after else 0),
+                                                 _stream()))
 
 
 def branch_norm_add_norm(x: torch.Tensor, branch: torch.Tensor, branch_weight: torch.Tensor, branch_eps: float,
@@ -644,6 +646,187 @@ def qkv_rotate_store(qkv: torch.Tensor, q_out: torch.Tensor, nh: int, nkv: int, 
         c_int(pv), c_int(1 if write_kv else 0), _stream()))
 
 
+def qkv_norm_rotate_store(qkv: torch.Tensor, q_out: torch.Tensor, nh: int, nkv: int, dk: int, dv: int, rot_dims: int,
+                          positions: torch.Tensor, tok_slot: torch.Tensor, inv_freq: Optional[torch.Tensor], mag: float,
+                          kpool: Optional[torch.Tensor], vpool: Optional[torch.Tensor],
+                          page_table: Optional[torch.Tensor], page_size: int, write_kv: bool = True,
+                          bias: Optional[torch.Tensor] = None, q_norm: Optional[torch.Tensor] = None,
+                          k_norm: Optional[torch.Tensor] = None, eps: float = 0.0, values_from_keys: bool = False):
+    """qkv_rotate_store with what some designs put between projection and rotation: ``bias`` (float32, as wide as
+    a row of qkv) is added; q heads and k heads are divided by their root mean square (eps inside the root) and
+    multiplied by a weight of dk numbers shared by the heads (q_norm, k_norm, float32 [dk]); with
+    values_from_keys a row is [q | k] only and the value pages receive k as projected (with its bias, before norm
+    and rotation)."""
+    ld = _ld(qkv, "qkv")
+    n = qkv.shape[0]
+    width = nh * dk + ((nkv * dk + (0 if values_from_keys else nkv * dv)) if write_kv else 0)
+    if qkv.shape[1] < width:
+        raise KernelError(f"qkv_norm_rotate_store: rows of {qkv.shape[1]} cannot hold {nh} query heads and {nkv} key/value heads")
+    if values_from_keys and dv != dk:
+        raise KernelError(f"qkv_norm_rotate_store: values that are the keys have the keys' size ({dv}, {dk})")
+    _need(q_out, "qkv q_out", qkv.dtype, (n, nh * dk))
+    _need(positions, "qkv positions", torch.int32, (n,))
+    if rot_dims:
+        _need(inv_freq, "qkv inv_freq", torch.float32, (rot_dims // 2,))
+    if bias is not None:
+        _need(bias, "qkv bias", torch.float32, (None,))
+        if bias.shape[0] < width:
+            raise KernelError(f"qkv_norm_rotate_store: a bias of {bias.shape[0]} numbers for rows of {width}")
+    for t, name in ((q_norm, "query norm weight"), (k_norm, "key norm weight")):
+        if t is not None:
+            _need(t, f"qkv {name}", torch.float32, (dk,))
+    tw = pk = pv = 0
+    if write_kv:
+        _need(tok_slot, "qkv token slots", torch.int32, (n,))
+        _need(page_table, "qkv page table", torch.int32, (None, None))
+        _need(kpool, "qkv key pool", qkv.dtype, (None, page_size, None))
+        _need(vpool, "qkv value pool", qkv.dtype, (kpool.shape[0], page_size, None))
+        if kpool.shape[2] % nkv or vpool.shape[2] % nkv:
+            raise KernelError(f"qkv_norm_rotate_store: pools of {kpool.shape[2]} / {vpool.shape[2]} features do not hold {nkv} heads")
+        tw, pk, pv = page_table.shape[1], kpool.shape[2] // nkv, vpool.shape[2] // nkv
+    _check(_fn("attention_general", "cpmcu_qkv_norm_rotate_store")(
+        _p(qkv), c_long(ld), c_int(_code(qkv)), _p(bias), _p(q_out), c_int(n), c_int(nh), c_int(nkv), c_int(dk), c_int(dv),
+        c_int(rot_dims), _p(q_norm), _p(k_norm), c_float(eps), c_int(1 if values_from_keys else 0), _p(positions),
+        _p(tok_slot), _p(inv_freq), c_float(mag), _p(kpool if write_kv else None), _p(vpool if write_kv else None),
+        _p(page_table if write_kv else None), c_int(tw), c_int(page_size), c_int(pk), c_int(pv),
+        c_int(1 if write_kv else 0), _stream()))
+
+
+def _parts_of(t: torch.Tensor, n: int, H: int, name: str):
+    """(parts, stride) of a branch [n, H] or of float partial sums [P, n, H]."""
+    if t.dim() == 3:
+        _need(t, name, shape=(None, n, H))
+        return t.shape[0], n * H
+    _need(t, name, shape=(n, H))
+    return 1, 0
+
+
+def gated_branches(gates: torch.Tensor, gate_bias: Optional[torch.Tensor], a: torch.Tensor, a_bias: Optional[torch.Tensor],
+                   f: Optional[torch.Tensor], f_bias: Optional[torch.Tensor], out: torch.Tensor):
+    """out = sigmoid(gates[:, :H] + gate_bias[:H]) * (a + a_bias) + sigmoid(gates[:, H:2H] + gate_bias[H:]) * (f + f_bias),
+    in float; a and f [n, H] or float partial sums [P, n, H]; f (with its gate) may be None.  gates may be a column
+    slice of a wider projection."""
+    _need(out, "gated out", torch.float32, (None, None))
+    n, H = out.shape
+    ldg = _ld(gates, "gates")
+    if gates.shape[0] != n or gates.shape[1] < (2 if f is not None else 1) * H:
+        raise KernelError(f"gated_branches: gates {tuple(gates.shape)} for {n} rows of {H}")
+    ap, astr = _parts_of(a, n, H, "gated branch")
+    fp, fstr = _parts_of(f, n, H, "gated second branch") if f is not None else (0, 0)
+    if gate_bias is not None:
+        _need(gate_bias, "gate bias", torch.float32, ((2 if f is not None else 1) * H,))
+    for t, name in ((a_bias, "branch bias"), (f_bias, "second branch bias")):
+        if t is not None:
+            _need(t, name, torch.float32, (H,))
+    _check(_fn("norms", "cpmcu_gated_branches")(
+        _p(gates), c_long(ldg), c_int(_code(gates)), _p(gate_bias), _p(a), c_int(_code(a)), c_int(ap), c_long(astr),
+        _p(a_bias), _p(f), c_int(_code(f) if f is not None else 0), c_int(fp), c_long(fstr), _p(f_bias), _p(out),
+        c_int(n), c_int(H), _stream()))
+
+
+def bias_sum(a: torch.Tensor, bias: torch.Tensor, out: torch.Tensor):
+    """out = a + bias in float, a [n, H] or float partial sums [P, n, H] (summed)."""
+    _need(out, "bias_sum out", torch.float32, (None, None))
+    n, H = out.shape
+    parts, stride = _parts_of(a, n, H, "bias_sum input")
+    _need(bias, "bias", torch.float32, (H,))
+    _check(_fn("norms", "cpmcu_bias_sum")(_p(a), c_int(_code(a)), c_int(parts), c_long(stride), _p(bias), _p(out),
+                                          c_int(n), c_int(H), _stream()))
+
+
+def mlstm_scan(proj: torch.Tensor, q_off: int, k_off: int, v_off: int, i_off: int, f_off: int, i_bias: torch.Tensor,
+               f_bias: torch.Tensor, cap: float, q_scale: float, S: torch.Tensor, n_state: torch.Tensor,
+               m_state: torch.Tensor, y: torch.Tensor, cu_q: torch.Tensor, seq_slot: torch.Tensor, heads: int, d: int,
+               dv: int, write_state: bool = True):
+    """The matrix-memory recurrence over each sequence's tokens, in float.  proj [n, W] holds, from the given
+    columns on, q and k (heads * d each), v (heads * dv) and the raw input and forget gates (heads each); per head
+    a = cap tanh((i + i_bias)/cap), b = logsigmoid(cap tanh((f + f_bias)/cap)), m' = max(b + m, a),
+    S' = exp(b + m - m') S + exp(a - m') k v^T, n' likewise with k, y = S'^T q / (max(|n'.q|, exp(-m')) + 1e-6),
+    q multiplied by q_scale.  S float32 [slots, heads, dv, d], n_state [slots, heads, d], m_state [slots, heads];
+    y float32 [n, heads * dv]."""
+    ld = _ld(proj, "mlstm projection")
+    n = proj.shape[0]
+    for off, w in ((q_off, heads * d), (k_off, heads * d), (v_off, heads * dv), (i_off, heads), (f_off, heads)):
+        if off < 0 or off + w > proj.shape[1]:
+            raise KernelError(f"mlstm_scan: columns {off}..{off + w} lie beyond rows of {proj.shape[1]}")
+    _need(i_bias, "mlstm input gate bias", torch.float32, (heads,))
+    _need(f_bias, "mlstm forget gate bias", torch.float32, (heads,))
+    _need(S, "mlstm state", torch.float32, (None, heads, dv, d))
+    _need(n_state, "mlstm normaliser", torch.float32, (S.shape[0], heads, d))
+    _need(m_state, "mlstm maximum", torch.float32, (S.shape[0], heads))
+    _need(y, "mlstm out", torch.float32, (n, heads * dv))
+    _need(cu_q, "mlstm sequence starts", torch.int32, (None,))
+    B = cu_q.shape[0] - 1
+    _need(seq_slot, "mlstm sequence slots", torch.int32, (B,))
+    _check(_fn("mlstm", "cpmcu_mlstm_scan")(_p(proj), c_long(ld), c_int(_code(proj)), c_long(q_off), c_long(k_off),
+                                            c_long(v_off), c_long(i_off), c_long(f_off), _p(i_bias), _p(f_bias),
+                                            c_float(cap), c_float(q_scale), _p(S), _p(n_state), _p(m_state), _p(y),
+                                            _p(cu_q), _p(seq_slot), c_int(B), c_int(heads), c_int(d), c_int(dv),
+                                            c_int(1 if write_state else 0), _stream()))
+
+
+MOE_MAX_EXPERTS = 1024
+
+
+def moe_route(h: torch.Tensor, router: torch.Tensor, correction: Optional[torch.Tensor], shared_gate: Optional[torch.Tensor],
+              n_groups: int, keep_groups: int, top: int, idx: torch.Tensor, weights: torch.Tensor,
+              shared_out: Optional[torch.Tensor] = None):
+    """Routing of every token to ``top`` of E experts.  Logits router . h in float (router float32 [E, H]), scores
+    s = softmax; choice scores s + correction; the experts form n_groups equal groups of neighbours, of which only
+    the keep_groups with the largest best choice score may be chosen from; the top largest choice scores win (ties:
+    the lower index); weights = s of the chosen / (their sum + 1e-20).  idx int32 [n, top], weights float32 [n, top].
+    shared_gate (float32 [H]): shared_out[t] = sigmoid(shared_gate . h[t])."""
+    ldh = _ld(h, "router input")
+    n, H = h.shape
+    _need(router, "router weight", torch.float32, (None, H))
+    E = router.shape[0]
+    if correction is not None:
+        _need(correction, "router correction", torch.float32, (E,))
+    if shared_gate is not None:
+        _need(shared_gate, "shared gate weight", torch.float32, (H,))
+        _need(shared_out, "shared gate", torch.float32, (n,))
+    _need(idx, "chosen experts", torch.int32, (n, top))
+    _need(weights, "expert weights", torch.float32, (n, top))
+    _check(_fn("moe", "cpmcu_moe_route")(_p(h), c_long(ldh), c_int(_code(h)), _p(router), _p(correction), _p(shared_gate),
+                                         c_int(n), c_int(H), c_int(E), c_int(n_groups), c_int(keep_groups), c_int(top),
+                                         _p(idx), _p(weights), _p(shared_out), _stream()))
+
+
+def moe_gated(h: torch.Tensor, gate_up: torch.Tensor, idx: torch.Tensor, act: torch.Tensor):
+    """act[t, k] = silu(Wg_e h[t]) * (Wu_e h[t]) for e = idx[t, k]; gate_up [E, 2F, H] (an expert's gate rows, then
+    its up rows), act [n, top, F], both of h's element type."""
+    ldh = _ld(h, "experts input")
+    n, H = h.shape
+    _need(gate_up, "experts gate/up", h.dtype, (None, None, H))
+    E, F2 = gate_up.shape[0], gate_up.shape[1]
+    if F2 % 2:
+        raise KernelError(f"moe_gated: {F2} stacked gate and up rows")
+    _need(idx, "chosen experts", torch.int32, (n, None))
+    top = idx.shape[1]
+    _need(act, "experts act", h.dtype, (n, top, F2 // 2))
+    _check(_fn("moe", "cpmcu_moe_gated")(_p(h), c_long(ldh), c_int(_code(h)), _p(gate_up), _p(idx), _p(act), c_int(n),
+                                         c_int(H), c_int(F2 // 2), c_int(top), _stream()))
+
+
+def moe_down(act: torch.Tensor, down: torch.Tensor, idx: torch.Tensor, weights: torch.Tensor, out: torch.Tensor,
+             shared: Optional[torch.Tensor] = None, shared_gate: Optional[torch.Tensor] = None):
+    """out[t] = sum_k weights[t, k] * Wd_e act[t, k] (+ shared_gate[t] * shared[t]); down [E, H, F]; out float32
+    [n, H]; shared [n, H] or float partial sums [P, n, H]."""
+    _need(act, "experts act", shape=(None, None, None))
+    n, top, F = act.shape
+    _need(down, "experts down", act.dtype, (None, None, F))
+    H = down.shape[1]
+    _need(idx, "chosen experts", torch.int32, (n, top))
+    _need(weights, "expert weights", torch.float32, (n, top))
+    _need(out, "experts out", torch.float32, (n, H))
+    sp, sstr = _parts_of(shared, n, H, "shared expert") if shared is not None else (0, 0)
+    if shared_gate is not None:
+        _need(shared_gate, "shared gate", torch.float32, (n,))
+    _check(_fn("moe", "cpmcu_moe_down")(_p(act), c_int(_code(act)), _p(down), _p(idx), _p(weights), _p(shared),
+                                        c_int(_code(shared) if shared is not None else 0), c_int(sp), c_long(sstr),
+                                        _p(shared_gate), _p(out), c_int(n), c_int(H), c_int(F), c_int(top), _stream()))
+
+
 def latent_store(proj: torch.Tensor, q_out: torch.Tensor, nh: int, dim: int, rot: int, rank: int,
                  norm_w: Optional[torch.Tensor], eps: float, positions: torch.Tensor, tok_slot: torch.Tensor,
                  inv_freq: Optional[torch.Tensor], mag: float, kpool: Optional[torch.Tensor],
@@ -679,10 +862,15 @@ def latent_store(proj: torch.Tensor, q_out: torch.Tensor, nh: int, dim: int, rot
 
 def attention_general(q: torch.Tensor, out: torch.Tensor, nh: int, nkv: int, hdk: int, hdv: int, scale: float,
                       kpool: torch.Tensor, vpool: torch.Tensor, page_table: torch.Tensor, page_size: int,
-                      positions: torch.Tensor, tok_slot: torch.Tensor, chunk: int = 0):
+                      positions: torch.Tensor, tok_slot: torch.Tensor, chunk: int = 0, window: int = 0,
+                      keep_first: int = 0, sink: Optional[torch.Tensor] = None):
     """Causal attention with key size hdk and value size hdv of their own (plain kernel, both element types).
     The cache may hold heads padded to a multiple of 16 features.  chunk > 0: the query at position p sees only
-    keys j <= p with j // chunk == p // chunk."""
+    keys j <= p with j // chunk == p // chunk.  window > 0: only keys with p - j < window, and the sequence's
+    first keep_first keys.  sink (float32 [nh]): exp(sink[h]) joins the softmax's denominator as a term without
+    a value."""
+    if sink is not None:
+        _need(sink, "attention sink", torch.float32, (nh,))
     _need(q, "attention q", shape=(None, nh * hdk))
     n = q.shape[0]
     _need(out, "attention out", q.dtype, (n, nh * hdv))
@@ -695,7 +883,8 @@ def attention_general(q: torch.Tensor, out: torch.Tensor, nh: int, nkv: int, hdk
     _need(tok_slot, "attention token slots", torch.int32, (n,))
     _check(_fn("attention_general", "cpmcu_attention_general")(
         _p(q), _p(out), c_int(_code(q)), c_int(n), c_int(nh), c_int(nkv), c_int(hdk), c_int(hdv),
-        c_int(kpool.shape[2] // nkv), c_int(vpool.shape[2] // nkv), c_float(scale), c_int(chunk), _p(kpool),
+        c_int(kpool.shape[2] // nkv), c_int(vpool.shape[2] // nkv), c_float(scale), c_int(chunk), c_int(window),
+        c_int(keep_first), _p(sink), _p(kpool),
         _p(vpool), _p(page_table), c_int(page_table.shape[1]), c_int(page_size), _p(positions), _p(tok_slot),
         _stream()))
 
@@ -1061,7 +1250,8 @@ def attention_general_mfma(q: torch.Tensor, out: torch.Tensor, nh: int, nkv: int
                            kpool: torch.Tensor, vpool: torch.Tensor, page_table: torch.Tensor, page_size: int,
                            positions: torch.Tensor, tok_slot: torch.Tensor, chunk: int = 0, n_splits: int = 1,
                            part_o: Optional[torch.Tensor] = None, part_ml: Optional[torch.Tensor] = None,
-                           tiles: Optional[torch.Tensor] = None, tokens_per_tile: int = 1):
+                           tiles: Optional[torch.Tensor] = None, tokens_per_tile: int = 1, window: int = 0,
+                           keep_first: int = 0, sink: Optional[torch.Tensor] = None):
     """attention_general in bf16 on the matrix cores (key size a multiple of 8 up to 1024, value size up to 512).
     With n_splits > 1 every token's visible keys are shared among n_splits workgroups and merged afterwards;
     part_o float32 [n, nh, n_splits, hdv] and part_ml float32 [n, nh, n_splits, 2] are its scratch.
@@ -1083,9 +1273,12 @@ def attention_general_mfma(q: torch.Tensor, out: torch.Tensor, nh: int, nkv: int
         _need(part_ml, "attention partial max/sum", torch.float32, (n, nh, n_splits, 2))
     if tiles is not None:
         _need(tiles, "attention tiles", torch.int32, (None, 2))
+    if sink is not None:
+        _need(sink, "attention sink", torch.float32, (nh,))
     _check(_fn("attention_general", "cpmcu_attention_general_mfma")(
         _p(q), _p(out), _p(part_o), _p(part_ml), c_int(n), c_int(nh), c_int(nkv), c_int(hdk), c_int(hdv),
-        c_int(kpool.shape[2] // nkv), c_int(vpool.shape[2] // nkv), c_float(scale), c_int(chunk), _p(kpool), _p(vpool),
+        c_int(kpool.shape[2] // nkv), c_int(vpool.shape[2] // nkv), c_float(scale), c_int(chunk), c_int(window),
+        c_int(keep_first), _p(sink), _p(kpool), _p(vpool),
         _p(page_table), c_int(page_table.shape[1]), c_int(page_size), _p(positions), _p(tok_slot), c_int(n_splits),
         _p(tiles), c_int(tiles.shape[0] if tiles is not None else 0), c_int(tokens_per_tile), _stream()))
 
@@ -1112,15 +1305,21 @@ def reserve_attention_general(ws, dtype, nh: int, nkv: int, hdv: int, pool_hdv: 
         ws.get("attn.gpart_ml", (most, nh, 2), torch.float32)
 
 
-def attention_any(q, out, nh, nkv, hdk, hdv, scale, kpool, vpool, page_table, page_size, ctx, chunk: int = 0):
-    """Attention with key and value sizes of their own and an optional chunked mask, with the kernel that suits
-    the step; writes ``out`` [n, nh*hdv]."""
-    if hdk == hdv and chunk == 0 and hdk <= 256 and kpool.shape[2] == nkv * hdk:
+def attention_any(q, out, nh, nkv, hdk, hdv, scale, kpool, vpool, page_table, page_size, ctx, chunk: int = 0,
+                  window: int = 0, keep_first: int = 0, sink: Optional[torch.Tensor] = None):
+    """Attention with key and value sizes of their own and an optional mask (chunks, or a sliding window with kept
+    first tokens) and softmax sink, with the kernel that suits the step; writes ``out`` [n, nh*hdv]."""
+    if (hdk == hdv and chunk == 0 and window == 0 and sink is None and hdk <= 256 and hdk % 16 == 0
+            and kpool.shape[2] == nkv * hdk):
         attention(q, out, nh, nkv, hdk, scale, kpool, vpool, page_table, page_size, ctx)
         return
     if attention_general_mfma_ok(q, hdk, hdv, page_size):
         n = q.shape[0]
-        keys = ctx.max_pos + 1 if chunk == 0 else min(ctx.max_pos + 1, chunk)
+        keys = ctx.max_pos + 1
+        if chunk:
+            keys = min(keys, chunk)
+        if window:
+            keys = min(keys, window + keep_first)
         splits = attention_general_splits(n, nkv, nh // nkv, vpool.shape[2] // nkv, keys) if ctx.single_token else 1
         part_o = part_ml = None
         if splits > 1:
@@ -1135,7 +1334,7 @@ def attention_any(q, out, nh, nkv, hdk, hdv, scale, kpool, vpool, page_table, pa
                 if tiles is None:
                     tiles = ctx.extras[key] = prefill_tiles(ctx.q_lens, tpt, q.device)
         attention_general_mfma(q, out, nh, nkv, hdk, hdv, scale, kpool, vpool, page_table, page_size, ctx.positions,
-                               ctx.tok_slot, chunk, splits, part_o, part_ml, tiles, tpt)
+                               ctx.tok_slot, chunk, splits, part_o, part_ml, tiles, tpt, window, keep_first, sink)
         return
     attention_general(q, out, nh, nkv, hdk, hdv, scale, kpool, vpool, page_table, page_size, ctx.positions,
-                      ctx.tok_slot, chunk)
+                      ctx.tok_slot, chunk, window, keep_first, sink)

@@ -7,6 +7,7 @@ from .rope import LongRotaryEncoding, RotaryEncoding, YarnRotaryEncoding
 from .attention import GeneralAttention, GQAAttention, InfLLMv2Attention
 from .latent_attention import LatentAttention
 from .ssm import Mamba2Mixer
-from .ffn import GatedFFN, PolyNormFFN
-from .block import PreNormBlock, SandwichNormBlock
+from .mlstm import MLSTMMixer
+from .ffn import GatedFFN, PolyNormFFN, RoutedExpertsFFN
+from .block import ParallelGatedBlock, PreNormBlock, SandwichNormBlock
 from .embedding import LMHead, TokenEmbedding

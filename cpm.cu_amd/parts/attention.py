@@ -23,7 +23,7 @@ import torch
 
 from .. import ops
 from ..cache.paged import CacheNeeds, CacheView, StreamSpec
-from .base import MIXERS, DeferredBranch, Mixer, Part, PositionEncoding, Runtime, StepContext
+from .base import MIXERS, BiasedBranch, DeferredBranch, Mixer, Part, PositionEncoding, Runtime, StepContext
 from .linear import Linear
 
 
@@ -224,39 +224,81 @@ def _pad16(n: int) -> int:
 class GeneralAttention(Mixer):
     """Grouped-query attention whose sizes are free: key size and value size of their own, a rotation that may
     cover only the first features of a head (the rest pass unchanged), a score scale from the configuration,
-    and an optional chunked mask: the query at position p sees key j <= p only if j // chunk == p // chunk,
-    chunks counted from position 0 of the sequence (not from where a prompt was cut).  Query head h reads kv head
-    h // (heads / kv_heads); no biases; softmax in float.  With a chunked mask the cache keeps a trailing window
-    of one chunk and gives older pages back.  ``names``: checkpoint tensors for 'q', 'k', 'v', 'out'."""
+    and an optional mask beyond the causal one: *chunked* (the query at position p sees key j <= p only if
+    j // chunk == p // chunk, chunks counted from position 0 of the sequence, not from where a prompt was cut), or
+    a *sliding window with kept first tokens* (key j <= p is seen if p - j < mask_window or j < mask_keep_first;
+    kept tokens keep their own positions).  Query head h reads kv head h // (heads / kv_heads); softmax in float.
+    With a mask the cache keeps a trailing window (and the kept first tokens' pages) and gives older pages back.
+
+    ``names``: checkpoint tensors for 'q', 'k', 'v', 'out', and optionally
+      'q_bias', 'k_bias', 'v_bias', 'out_bias'  biases of the projections (added in float by the kernel that reads
+                                                 the product);
+      'q_norm', 'k_norm'   weights of dk numbers, shared by the heads: q and k heads are divided by their root mean
+                           square (``norm_eps`` inside the root) and multiplied by them before the rotation;
+      'sink'               one number a head: exp(sink) joins the softmax's denominator as a term that has no key,
+                           no value and no scale.
+    Without 'v' the values are the keys as projected (with their bias, before norm and rotation): value_dim
+    must equal key_dim."""
 
     def __init__(self, names: Mapping[str, str], hidden_size: int, num_heads: int, num_kv_heads: int, key_dim: int,
-                 value_dim: int, position: Optional[PositionEncoding], scale: float, mask_chunk: Optional[int] = None):
+                 value_dim: int, position: Optional[PositionEncoding], scale: float, mask_chunk: Optional[int] = None,
+                 mask_window: Optional[int] = None, mask_keep_first: int = 0, norm_eps: float = 0.0):
         if num_heads % num_kv_heads:
             raise ValueError(f"attention: {num_heads} heads are not a multiple of {num_kv_heads} kv heads")
         if key_dim > 1024 or value_dim > 1024:
             raise ValueError(f"attention: key size {key_dim} / value size {value_dim} exceed the kernel's 1024")
         if mask_chunk is not None and mask_chunk <= 0:
             raise ValueError(f"attention: a mask chunk of {mask_chunk} tokens")
+        if mask_window is not None and mask_window <= 0:
+            raise ValueError(f"attention: a mask window of {mask_window} tokens")
+        if mask_chunk and mask_window:
+            raise ValueError("attention: a chunked mask or a sliding window, not both")
+        if mask_keep_first < 0 or (mask_keep_first and not mask_window):
+            raise ValueError("attention: kept first tokens come with a sliding window")
         self.names = dict(names)
+        self.values_are_keys = "v" not in self.names
+        if self.values_are_keys and value_dim != key_dim:
+            raise ValueError(f"attention: values that are the keys have the keys' size ({value_dim}, {key_dim})")
         self.hidden_size, self.nh, self.nkv, self.dk, self.dv = hidden_size, num_heads, num_kv_heads, key_dim, value_dim
         self.position, self.scale, self.chunk = position, float(scale), int(mask_chunk or 0)
-        self.qkv = Linear([(self.names["q"], num_heads * key_dim), (self.names["k"], num_kv_heads * key_dim),
-                           (self.names["v"], num_kv_heads * value_dim)], hidden_size)
-        self.o = Linear([(self.names["out"], hidden_size)], num_heads * value_dim)
+        self.window, self.keep_first, self.norm_eps = int(mask_window or 0), int(mask_keep_first), float(norm_eps)
+        stacked = [(self.names["q"], num_heads * key_dim), (self.names["k"], num_kv_heads * key_dim)]
+        biases = [self.names.get("q_bias"), self.names.get("k_bias")]
+        if not self.values_are_keys:
+            stacked.append((self.names["v"], num_kv_heads * value_dim))
+            biases.append(self.names.get("v_bias"))
+        self.qkv = Linear(stacked, hidden_size, bias_names=biases if any(biases) else None)
+        self.o = Linear([(self.names["out"], hidden_size)], num_heads * value_dim,
+                        bias_names=[self.names["out_bias"]] if self.names.get("out_bias") else None)
+        # what the plain rotate-and-store kernel does not do
+        self._extras = bool(any(biases) or self.names.get("q_norm") or self.names.get("k_norm") or self.values_are_keys)
 
     def parts(self) -> List[Part]:
         return [self.qkv, self.o] + ([self.position] if self.position is not None else [])
 
+    def weight_specs(self):
+        from .base import WeightSpec
+        specs = [WeightSpec(self.names[k], (self.dk,), "norm") for k in ("q_norm", "k_norm") if self.names.get(k)]
+        if self.names.get("sink"):
+            specs.append(WeightSpec(self.names["sink"], (self.nh,), "small"))
+        return specs
+
     def bind(self, tensors: Mapping[str, torch.Tensor], rt: Runtime):
         self.rt = rt
+        f = lambda k: tensors[self.names[k]].to(torch.float32).contiguous() if self.names.get(k) else None
+        self.q_norm, self.k_norm, self.sink = f("q_norm"), f("k_norm"), f("sink")
 
     def cache_needs(self) -> CacheNeeds:
         return CacheNeeds(streams=(("k", StreamSpec(self.nkv * _pad16(self.dk))),
                                    ("v", StreamSpec(self.nkv * _pad16(self.dv)))),
-                          window=self.chunk or None)
+                          window=self.chunk or self.window or None, keep_first=self.keep_first)
 
     def reserve_workspace(self, ws, rt: Runtime, max_step_tokens: int, max_slots: int):
-        keys = min(rt.max_seq_len, self.chunk) if self.chunk else rt.max_seq_len
+        keys = rt.max_seq_len
+        if self.chunk:
+            keys = min(keys, self.chunk)
+        if self.window:
+            keys = min(keys, self.window + self.keep_first)
         ops.reserve_attention_general(ws, rt.dtype, self.nh, self.nkv, self.dv, _pad16(self.dv), keys, max_step_tokens)
 
     def forward(self, h, ctx: StepContext, cache: CacheView, writes_cache: bool = True):
@@ -271,12 +313,20 @@ class GeneralAttention(Mixer):
         with ctx.timed("attn_qkv_rope"):
             qkv = self.qkv.forward(h, ctx, "attn.qkv", rows=None if writes_cache else nh * dk)
             q = ctx.ws.get("attn.q", (n, nh * dk), self.rt.dtype)
-            ops.qkv_rotate_store(qkv, q, nh, nkv, dk, dv, rd, ctx.positions, ctx.tok_slot, inv_freq, mag,
-                                 cache.streams["k"], cache.streams["v"], cache.page_table, cache.page_size,
-                                 write_kv=writes_cache)
+            if self._extras:
+                ops.qkv_norm_rotate_store(qkv, q, nh, nkv, dk, dv, rd, ctx.positions, ctx.tok_slot, inv_freq, mag,
+                                          cache.streams["k"], cache.streams["v"], cache.page_table, cache.page_size,
+                                          write_kv=writes_cache, bias=self.qkv.bias, q_norm=self.q_norm,
+                                          k_norm=self.k_norm, eps=self.norm_eps, values_from_keys=self.values_are_keys)
+            else:
+                ops.qkv_rotate_store(qkv, q, nh, nkv, dk, dv, rd, ctx.positions, ctx.tok_slot, inv_freq, mag,
+                                     cache.streams["k"], cache.streams["v"], cache.page_table, cache.page_size,
+                                     write_kv=writes_cache)
         out = ctx.ws.get("attn.out", (n, nh * dv), self.rt.dtype)
         with ctx.timed("attn_core"):
             ops.attention_any(q, out, nh, nkv, dk, dv, self.scale, cache.streams["k"], cache.streams["v"],
-                              cache.page_table, cache.page_size, ctx, chunk=self.chunk)
+                              cache.page_table, cache.page_size, ctx, chunk=self.chunk, window=self.window,
+                              keep_first=self.keep_first, sink=self.sink)
         with ctx.timed("attn_o"):
-            return self.o.forward(out, ctx, "attn.o", out_dtype=torch.float32, partials=True)
+            branch = self.o.forward(out, ctx, "attn.o", out_dtype=torch.float32, partials=True)
+        return BiasedBranch(branch, self.o.bias, ctx, "attn.o") if self.o.bias is not None else branch

@@ -17,7 +17,8 @@ Kinds of parts and what each must provide:
 * ``Block``:     forward(stream, ctx, cache, writes_cache): the arrangement of the above
                  around the residual stream
 
-A branch may have a norm of its own before it joins the residual (``NormedBranch``; ``Norm.normalize``).
+A branch may have a norm of its own before it joins the residual (``NormedBranch``; ``Norm.normalize``), or a
+bias that its consumer adds (``BiasedBranch``).
 
 Two optional protocols let neighbouring parts share a kernel without knowing each other: a norm may leave
 its row factor to the product that follows (``forward_unscaled`` / ``takes_row_scale``), and a part may leave
@@ -170,9 +171,28 @@ class NormedBranch:
         return self._value
 
 
+class BiasedBranch:
+    """A branch whose last product has a bias that is not added yet: branch = ``branch`` + ``bias`` (float32 [H]),
+    ``branch`` a tensor [n, H] or float partial sums [P, n, H].  A consumer that adds the bias in a kernel of its
+    own takes the two as they are (a parallel layer's gate kernel does; ``Norm.takes_biased_branch``); for
+    everybody else ``evaluate()`` gives the float sum."""
+
+    def __init__(self, branch: torch.Tensor, bias: torch.Tensor, ctx: "StepContext", tag: str):
+        self.branch, self.bias, self.ctx, self.tag = branch, bias, ctx, tag
+        self._value: Optional[torch.Tensor] = None
+
+    def evaluate(self) -> torch.Tensor:
+        if self._value is None:
+            from .. import ops
+            n, H = self.branch.shape[-2], self.branch.shape[-1]
+            self._value = self.ctx.ws.get(self.tag + ".biased", (n, H), torch.float32)
+            ops.bias_sum(self.branch, self.bias, self._value)
+        return self._value
+
+
 def branch_tensor(branch):
     """The branch as a tensor (or None), whatever form it was handed over in."""
-    return branch.evaluate() if isinstance(branch, (DeferredBranch, NormedBranch)) else branch
+    return branch.evaluate() if isinstance(branch, (DeferredBranch, NormedBranch, BiasedBranch)) else branch
 
 
 def branch_for(norm: "Norm", branch):
@@ -181,6 +201,8 @@ def branch_for(norm: "Norm", branch):
     if isinstance(branch, DeferredBranch) and not norm.takes_deferred_branch:
         return branch.evaluate()
     if isinstance(branch, NormedBranch) and not norm.takes_normed_branch:
+        return branch.evaluate()
+    if isinstance(branch, BiasedBranch) and not norm.takes_biased_branch:
         return branch.evaluate()
     return branch
 
@@ -269,6 +291,8 @@ class Norm(Part):
     takes_deferred_branch = False
     # True if forward and forward_unscaled accept a NormedBranch as ``branch``
     takes_normed_branch = False
+    # True if forward and forward_unscaled accept a BiasedBranch as ``branch``
+    takes_biased_branch = False
 
     def normalize(self, t: torch.Tensor, ctx: StepContext, tag: str = "norm.plain") -> torch.Tensor:
         """The norm of the rows of ``t`` alone, float32 [n, H]: no residual, nothing added (what a branch that

@@ -11,8 +11,12 @@ from __future__ import annotations
 from typing import List, Optional
 
 from ..cache.paged import CacheView
-from .base import (BLOCKS, Block, DeferredBranch, FeedForward, Mixer, Norm, NormedBranch, Part, ResidualStream,
-                   StepContext, branch_for, forward_declares)
+import torch
+
+from .. import ops
+from .base import (BLOCKS, BiasedBranch, Block, DeferredBranch, FeedForward, Mixer, Norm, NormedBranch, Part,
+                   ResidualStream, StepContext, branch_for, branch_tensor, forward_declares)
+from .linear import Linear
 
 
 @BLOCKS.register("pre_norm")
@@ -107,4 +111,50 @@ class SandwichNormBlock(Block):
                 with ctx.timed("norm"):
                     h = self.ff_norm.forward(stream.x, branch_for(self.ff_norm, a), 1.0, ctx, tag="block.h")
                 stream.pending = NormedBranch(self.feed_forward.forward(h, ctx), self.ff_post_norm, ctx, "block.post")
+        stream.pending_scale = 1.0
+
+
+@BLOCKS.register("parallel_gated")
+class ParallelGatedBlock(Block):
+    """One norm a layer, both sub-layers read its output, and each sub-layer's result passes a gate that is a
+    projection of the same rows: with h = norm(x),
+
+        x += sigmoid(G1 h + g1) * Mixer(h) + sigmoid(G2 h + g2) * FeedForward(h)
+
+    element by element.  A layer may have no feed-forward (the second term and its gate are then absent).  The
+    two gates are one stacked product; the sum is left pending (float) for the norm that follows.
+    ``gate_names``: checkpoint tensors (weight, bias) of the mixer's gate and, with a feed-forward, of its gate."""
+
+    def __init__(self, norm: Norm, mixer: Mixer, feed_forward: Optional[FeedForward], hidden_size: int,
+                 gate_names: List[tuple]):
+        if len(gate_names) != (2 if feed_forward is not None else 1):
+            raise ValueError("parallel_gated: one gate (weight, bias) for every sub-layer")
+        self.norm, self.mixer, self.feed_forward, self.hidden_size = norm, mixer, feed_forward, hidden_size
+        self.gates = Linear([(w, hidden_size) for w, _ in gate_names], hidden_size, bias_names=[b for _, b in gate_names])
+
+    def parts(self) -> List[Part]:
+        return [self.norm, self.mixer] + ([self.feed_forward] if self.feed_forward is not None else []) + [self.gates]
+
+    @staticmethod
+    def _with_bias(branch):
+        if isinstance(branch, BiasedBranch):
+            return branch.branch, branch.bias
+        return branch_tensor(branch), None
+
+    def forward(self, stream: ResidualStream, ctx: StepContext, cache: Optional[CacheView], writes_cache: bool = True):
+        with ctx.timed("norm"):
+            h = self.norm.forward(stream.x, branch_for(self.norm, stream.take_pending()), stream.pending_scale, ctx,
+                                  tag="block.h")
+        with ctx.timed("attn"):
+            a, a_bias = self._with_bias(self.mixer.forward(h, ctx, cache, writes_cache))
+        f = f_bias = None
+        if self.feed_forward is not None:
+            with ctx.timed("ffn"):
+                f, f_bias = self._with_bias(self.feed_forward.forward(h, ctx))
+        with ctx.timed("gates"):
+            few = h.shape[0] <= ops.SKINNY_MAX_ROWS
+            g = self.gates.forward(h, ctx, "block.gates", out_dtype=torch.float32 if few else None)
+            out = ctx.ws.get("block.gated", (h.shape[0], self.hidden_size), torch.float32)
+            ops.gated_branches(g, self.gates.bias, a, a_bias, f, f_bias, out)
+        stream.pending = out
         stream.pending_scale = 1.0

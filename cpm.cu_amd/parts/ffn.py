@@ -5,7 +5,7 @@ gate and up are one stacked product, gate rows first (src/model/ffn.cuh:31-59,
 """
 from __future__ import annotations
 
-from typing import List, Mapping
+from typing import List, Mapping, Optional, Tuple
 
 import torch
 
@@ -16,12 +16,15 @@ from .linear import Linear
 
 @FEED_FORWARDS.register("gated_silu")
 class GatedFFN(FeedForward):
-    def __init__(self, prefix: str, hidden_size: int, intermediate_size: int):
+    def __init__(self, prefix: str, hidden_size: int, intermediate_size: int, names: Optional[Mapping[str, str]] = None):
+        """``names``: the checkpoint tensors for 'gate', 'up', 'down' behind the prefix (default: the MiniCPM
+        checkpoint's gate_proj.weight, up_proj.weight, down_proj.weight)."""
         self.hidden_size = hidden_size
         self.intermediate_size = intermediate_size
-        self.gate_up = Linear([(prefix + "gate_proj.weight", intermediate_size),
-                               (prefix + "up_proj.weight", intermediate_size)], hidden_size)
-        self.down = Linear([(prefix + "down_proj.weight", hidden_size)], intermediate_size)
+        names = names or {"gate": "gate_proj.weight", "up": "up_proj.weight", "down": "down_proj.weight"}
+        self.gate_up = Linear([(prefix + names["gate"], intermediate_size),
+                               (prefix + names["up"], intermediate_size)], hidden_size)
+        self.down = Linear([(prefix + names["down"], hidden_size)], intermediate_size)
 
     def parts(self) -> List[Part]:
         return [self.gate_up, self.down]
@@ -73,3 +76,82 @@ class PolyNormFFN(FeedForward):
             ops.poly_norm(z, self.coef, self.eps, act)
         with ctx.timed("ffn_down"):
             return self.down.forward(act, ctx, "ffn.down", out_dtype=torch.float32, partials=True)
+
+
+@FEED_FORWARDS.register("routed_experts")
+class RoutedExpertsFFN(FeedForward):
+    """A mixture of small SiLU-gated feed-forwards (no biases), of which every token uses ``top``.
+
+    Router: logits z = W_router h in float, scores s = softmax(z) over all experts.  The choice goes by s + a
+    correction a expert (a checkpoint tensor; the weights use s without it).  With ``groups`` = (count, keep) the
+    experts form ``count`` equal groups of neighbours, a group's score is its largest choice score, and only experts
+    of the ``keep`` best groups can be chosen.  The chosen experts' outputs are added with weights s / (sum of the
+    chosen s + 1e-20).  A shared expert (``shared_size``) runs for every token and is added times sigmoid(w . h),
+    one number a token.
+
+    ``names``: 'router', 'correction' (or absent), 'expert' (a format with {e} for the expert's number and {part}
+    for gate / up / down), and for the shared expert 'shared_gate', 'shared_up', 'shared_down', 'shared_scale'."""
+
+    def __init__(self, names: Mapping[str, str], hidden_size: int, expert_size: int, experts: int, top: int,
+                 groups: Optional[Tuple[int, int]] = None, shared_size: Optional[int] = None):
+        if experts > ops.MOE_MAX_EXPERTS:
+            raise ValueError(f"routed_experts: {experts} experts (up to {ops.MOE_MAX_EXPERTS} are taken)")
+        if not 0 < top <= experts:
+            raise ValueError(f"routed_experts: {top} of {experts} experts a token")
+        if groups is not None:
+            count, keep = groups
+            if count <= 0 or experts % count or not 0 < keep <= count or top > keep * (experts // count):
+                raise ValueError(f"routed_experts: {experts} experts in {count} groups, {keep} kept, {top} chosen")
+        self.names = dict(names)
+        self.hidden_size, self.expert_size, self.experts, self.top = hidden_size, expert_size, experts, top
+        self.groups = tuple(groups) if groups is not None else (1, 1)
+        self.shared = None
+        if shared_size is not None:
+            self.shared = GatedFFN("", hidden_size, shared_size, names={"gate": self.names["shared_gate"],
+                                                                        "up": self.names["shared_up"],
+                                                                        "down": self.names["shared_down"]})
+
+    def _expert(self, e: int, part: str) -> str:
+        return self.names["expert"].format(e=e, part=part)
+
+    def parts(self) -> List[Part]:
+        return [self.shared] if self.shared is not None else []
+
+    def weight_specs(self) -> List[WeightSpec]:
+        H, F = self.hidden_size, self.expert_size
+        specs = [WeightSpec(self.names["router"], (self.experts, H))]
+        if self.names.get("correction"):
+            specs.append(WeightSpec(self.names["correction"], (self.experts,), "small"))
+        for e in range(self.experts):
+            specs += [WeightSpec(self._expert(e, "gate"), (F, H)), WeightSpec(self._expert(e, "up"), (F, H)),
+                      WeightSpec(self._expert(e, "down"), (H, F))]
+        if self.shared is not None:
+            specs.append(WeightSpec(self.names["shared_scale"], (1, H)))
+        return specs
+
+    def bind(self, tensors: Mapping[str, torch.Tensor], rt: Runtime):
+        self.rt = rt
+        f32 = lambda name: tensors[name].to(torch.float32).contiguous()
+        self.router = f32(self.names["router"])
+        self.correction = f32(self.names["correction"]) if self.names.get("correction") else None
+        self.shared_scale = f32(self.names["shared_scale"]).reshape(-1) if self.shared is not None else None
+        # an expert's gate rows, then its up rows: [E, 2F, H]; down: [E, H, F]
+        self.gate_up = torch.stack([torch.cat([tensors[self._expert(e, "gate")], tensors[self._expert(e, "up")]], 0)
+                                    for e in range(self.experts)]).to(rt.dtype).contiguous()
+        self.down = torch.stack([tensors[self._expert(e, "down")] for e in range(self.experts)]).to(rt.dtype).contiguous()
+
+    def forward(self, h: torch.Tensor, ctx: StepContext):
+        n = h.shape[0]
+        idx = ctx.ws.get("moe.idx", (n, self.top), torch.int32)
+        wts = ctx.ws.get("moe.weights", (n, self.top), torch.float32)
+        sg = ctx.ws.get("moe.shared_gate", (n,), torch.float32) if self.shared is not None else None
+        with ctx.timed("moe_route"):
+            ops.moe_route(h, self.router, self.correction, self.shared_scale, self.groups[0], self.groups[1], self.top,
+                          idx, wts, sg)
+        shared = self.shared.forward(h, ctx) if self.shared is not None else None
+        act = ctx.ws.get("moe.act", (n, self.top, self.expert_size), self.rt.dtype)
+        out = ctx.ws.get("moe.out", (n, self.hidden_size), torch.float32)
+        with ctx.timed("moe_experts"):
+            ops.moe_gated(h, self.gate_up, idx, act)
+            ops.moe_down(act, self.down, idx, wts, out, shared, sg)
+        return out

@@ -16,21 +16,37 @@ from .base import Part, Runtime, StepContext, WeightSpec
 
 
 class Linear(Part):
-    def __init__(self, names: Sequence[Tuple[str, int]], in_features: int, init: str = "matrix"):
+    """``bias_names``: one checkpoint tensor (or None) for each stacked weight.  The product itself adds no bias:
+    ``bias`` (float32 [out], zeros where a stacked weight has none) is there for the kernel that consumes the
+    product (a rotation, a gate, a residual add), which adds it in float."""
+
+    def __init__(self, names: Sequence[Tuple[str, int]], in_features: int, init: str = "matrix",
+                 bias_names: Optional[Sequence[Optional[str]]] = None):
         self.names = list(names)
         self.in_features = in_features
         self.out_features = sum(r for _, r in self.names)
         self.init = init
         self.weight: Optional[torch.Tensor] = None
+        self.bias_names = list(bias_names) if bias_names is not None else None
+        if self.bias_names is not None and len(self.bias_names) != len(self.names):
+            raise ValueError("linear: a bias name (or None) is needed for each stacked weight")
+        self.bias: Optional[torch.Tensor] = None
 
     def weight_specs(self) -> List[WeightSpec]:
-        return [WeightSpec(n, (r, self.in_features), self.init) for n, r in self.names]
+        specs = [WeightSpec(n, (r, self.in_features), self.init) for n, r in self.names]
+        if self.bias_names is not None:
+            specs += [WeightSpec(b, (r,), "small") for b, (_, r) in zip(self.bias_names, self.names) if b is not None]
+        return specs
 
     def bind(self, tensors: Mapping[str, torch.Tensor], rt: Runtime):
         ws = [tensors[n] for n, _ in self.names]
         w = ws[0] if len(ws) == 1 else torch.cat(ws, dim=0)
         self.weight = w.to(rt.dtype).contiguous()
         self.rt = rt
+        if self.bias_names is not None and any(b is not None for b in self.bias_names):
+            self.bias = torch.cat([tensors[b].to(torch.float32) if b is not None
+                                   else torch.zeros(r, dtype=torch.float32, device=w.device)
+                                   for b, (_, r) in zip(self.bias_names, self.names)]).contiguous()
         # a second copy laid out for the decode product (bf16 engine; costs the weight's size again)
         self.tiled = ops.TiledWeight(self.weight) if (rt.dtype == torch.bfloat16 and rt.tiled_weights) else None
 

@@ -16,19 +16,24 @@ from .base import NORMS, DeferredBranch, Norm, NormedBranch, Runtime, StepContex
 
 @NORMS.register("rms_norm")
 class RMSNorm(Norm):
-    """``unit_offset``: the checkpoint stores the weight around zero and the norm multiplies by 1 + w."""
+    """``unit_offset``: the checkpoint stores the weight around zero and the norm multiplies by 1 + w.
+    ``scalar``: the checkpoint holds one number (a tensor without axes) that multiplies every coordinate."""
 
-    def __init__(self, name: str, hidden_size: int, eps: float, unit_offset: bool = False):
+    def __init__(self, name: str, hidden_size: int, eps: float, unit_offset: bool = False, scalar: bool = False):
         self.name = name
         self.hidden_size = hidden_size
         self.eps = float(eps)
         self.unit_offset = bool(unit_offset)
+        self.scalar = bool(scalar)
 
     def weight_specs(self) -> List[WeightSpec]:
-        return [WeightSpec(self.name, (self.hidden_size,), "norm_offset" if self.unit_offset else "norm")]
+        return [WeightSpec(self.name, () if self.scalar else (self.hidden_size,),
+                           "norm_offset" if self.unit_offset else "norm")]
 
     def bind(self, tensors: Mapping[str, torch.Tensor], rt: Runtime):
         w = tensors[self.name].to(torch.float32)
+        if self.scalar:
+            w = w.reshape(1).expand(self.hidden_size)
         self.weight = (w + 1.0 if self.unit_offset else w).contiguous()
         self.rt = rt
 
