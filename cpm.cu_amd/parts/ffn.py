@@ -121,7 +121,7 @@ class RoutedExpertsFFN(FeedForward):
         H, F = self.hidden_size, self.expert_size
         specs = [WeightSpec(self.names["router"], (self.experts, H))]
         if self.names.get("correction"):
-            specs.append(WeightSpec(self.names["correction"], (self.experts,), "small"))
+            specs.append(WeightSpec(self.names["correction"], (self.experts,), "slight"))
         for e in range(self.experts):
             specs += [WeightSpec(self._expert(e, "gate"), (F, H)), WeightSpec(self._expert(e, "up"), (F, H)),
                       WeightSpec(self._expert(e, "down"), (H, F))]

@@ -75,6 +75,12 @@ def _init_small(spec, g, device, dtype, std, norm_std):
     return (torch.randn(spec.shape, generator=g, dtype=torch.float32, device=device) * 0.5).to(dtype)
 
 
+@register_init_rule("slight")
+def _init_slight(spec, g, device, dtype, std, norm_std):
+    """N(0, 0.05): a correction added to softmax scores, which must shift a choice now and then, not make it."""
+    return (torch.randn(spec.shape, generator=g, dtype=torch.float32, device=device) * 0.05).to(dtype)
+
+
 @register_init_rule("conv_taps")
 def _init_conv_taps(spec, g, device, dtype, std, norm_std):
     """N(0, 1/sqrt(taps)): the taps of a short convolution per channel."""
