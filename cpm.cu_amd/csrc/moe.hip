@@ -260,3 +260,210 @@ extern "C" const char* cpmcu_moe_down(const void* act, int dtype, const void* wd
     CPMCU_LAUNCH_CHECK("moe_down");
     return nullptr;
 }
+
+// ===========================================================================
+// The same experts for steps of many tokens, bf16 on the matrix cores (v_mfma_f32_16x16x32_bf16): the (token,
+// chosen expert) pairs are grouped by expert into tiles of 64 rows, and every tile is a product with its
+// expert's weights.
+//
+//  * moe_group_kernel (one workgroup): counts the pairs of every expert, gives every expert whole tiles of 64 rows
+//    (rows[tile * 64 + i] = pair, -1 in a tile's unused rows), tile_expert[tile] and the number of tiles.  Which row
+//    of its expert's tiles a pair gets depends on timing; its result does not (a row's sums are its own).
+//  * moe_gated_mfma_kernel: act[pair] = silu(Wg_e h_t) * (Wu_e h_t); a wavefront owns 16 rows of a tile and 32
+//    features (two tiles of gate rows, two of up rows), operands straight from memory.
+//  * moe_down_mfma_kernel: y[pair] = Wd_e act[pair] (bf16); a wavefront owns 16 rows and 64 columns.
+//  * moe_combine_kernel: out[t] = sum_k w[t, k] y[t, k] (+ sg[t] * shared[t]) in float, k in order.
+// ===========================================================================
+typedef __bf16 mbf16x8_t __attribute__((ext_vector_type(8)));
+typedef float mfloatx4_t __attribute__((ext_vector_type(4)));
+
+#define MOE_TILE 64
+
+__global__ __launch_bounds__(1024) void moe_group_kernel(const int* __restrict__ idx, int n_pairs, int E,
+                                                         int* __restrict__ rows, int* __restrict__ tile_expert,
+                                                         int* __restrict__ n_tiles_out, int max_tiles) {
+    __shared__ int counts[MOE_MAX_EXPERTS];
+    __shared__ int offs[MOE_MAX_EXPERTS];
+    for (int e = threadIdx.x; e < E; e += 1024) counts[e] = 0;
+    for (int i = threadIdx.x; i < max_tiles * MOE_TILE; i += 1024) rows[i] = -1;
+    __syncthreads();
+    for (int p = threadIdx.x; p < n_pairs; p += 1024) atomicAdd(&counts[idx[p]], 1);
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        int t = 0;
+        for (int e = 0; e < E; ++e) {
+            offs[e] = t * MOE_TILE;
+            const int nt = (counts[e] + MOE_TILE - 1) / MOE_TILE;
+            for (int i = 0; i < nt; ++i) tile_expert[t + i] = e;
+            t += nt;
+        }
+        *n_tiles_out = t;
+    }
+    __syncthreads();
+    for (int e = threadIdx.x; e < E; e += 1024) counts[e] = 0;
+    __syncthreads();
+    for (int p = threadIdx.x; p < n_pairs; p += 1024) {
+        const int e = idx[p];
+        rows[offs[e] + atomicAdd(&counts[e], 1)] = p;
+    }
+}
+
+// grid (ceil(F / 32), max_tiles), 256 threads
+__global__ __launch_bounds__(256) void moe_gated_mfma_kernel(const bf16_t* __restrict__ h, long ldh,
+                                                             const bf16_t* __restrict__ wgu, const int* __restrict__ rows,
+                                                             const int* __restrict__ tile_expert,
+                                                             const int* __restrict__ n_tiles, bf16_t* __restrict__ act,
+                                                             int H, int F, int top) {
+    const int tile = blockIdx.y;
+    if (tile >= *n_tiles) return;
+    const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    const int lane = threadIdx.x & 63, r = lane & 15, g = lane >> 4;
+    const int e = tile_expert[tile];
+    const int f0 = blockIdx.x * 32;
+    const int pair = rows[tile * MOE_TILE + wave * 16 + r];
+    const bool row_ok = pair >= 0;
+    const bf16_t* xp = h + (long)(row_ok ? pair / top : 0) * ldh + g * 8;
+    const bf16_t* wp = wgu + (long)e * 2 * F * H + g * 8;
+    mfloatx4_t acc[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) acc[j] = mfloatx4_t{0.f, 0.f, 0.f, 0.f};
+    long wrow[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {                 // j = 0, 1: gate rows f0 + 16 j + r; j = 2, 3: their up rows
+        const int f = min(f0 + 16 * (j & 1) + r, F - 1);
+        wrow[j] = (long)((j >> 1) * F + f) * H;
+    }
+#pragma unroll 2
+    for (int k0 = 0; k0 < H; k0 += 32) {
+        const bool k_ok = k0 + g * 8 < H;
+        const int kk = k_ok ? k0 : k0 - g * 8;       // a lane beyond the row's end reads the step's first columns (in range) and is zeroed
+        mbf16x8_t a = *(const mbf16x8_t*)(xp + kk);
+        mbf16x8_t b[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) b[j] = *(const mbf16x8_t*)(wp + wrow[j] + kk);
+        if (!k_ok) {
+            a = mbf16x8_t{0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+            for (int j = 0; j < 4; ++j) b[j] = a;
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b[j], acc[j], 0, 0, 0);
+    }
+    // lane (feature column r, g): acc[j][i] belongs to the tile's row wave * 16 + 4 g + i
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int p = rows[tile * MOE_TILE + wave * 16 + 4 * g + i];
+        if (p < 0) continue;
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const int f = f0 + 16 * j + r;
+            if (f < F) {
+                const float gt = acc[j][i], up = acc[2 + j][i];
+                act[(long)p * F + f] = f32_to_bf16(gt / (1.0f + expf(-gt)) * up);
+            }
+        }
+    }
+}
+
+// grid (ceil(H / 64), max_tiles), 256 threads
+__global__ __launch_bounds__(256) void moe_down_mfma_kernel(const bf16_t* __restrict__ act, const bf16_t* __restrict__ wd,
+                                                            const int* __restrict__ rows,
+                                                            const int* __restrict__ tile_expert,
+                                                            const int* __restrict__ n_tiles, bf16_t* __restrict__ y,
+                                                            int H, int F) {
+    const int tile = blockIdx.y;
+    if (tile >= *n_tiles) return;
+    const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
+    const int lane = threadIdx.x & 63, r = lane & 15, g = lane >> 4;
+    const int e = tile_expert[tile];
+    const int c0 = blockIdx.x * 64;
+    const int pair = rows[tile * MOE_TILE + wave * 16 + r];
+    const bf16_t* xp = act + (long)(pair >= 0 ? pair : 0) * F + g * 8;
+    const bf16_t* wp = wd + (long)e * H * F + g * 8;
+    mfloatx4_t acc[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) acc[j] = mfloatx4_t{0.f, 0.f, 0.f, 0.f};
+    long wrow[4];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) wrow[j] = (long)min(c0 + 16 * j + r, H - 1) * F;
+#pragma unroll 2
+    for (int k0 = 0; k0 < F; k0 += 32) {
+        const bool k_ok = k0 + g * 8 < F;
+        const int kk = k_ok ? k0 : k0 - g * 8;       // a lane beyond the row's end reads the step's first columns (in range) and is zeroed
+        mbf16x8_t a = *(const mbf16x8_t*)(xp + kk);
+        mbf16x8_t b[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) b[j] = *(const mbf16x8_t*)(wp + wrow[j] + kk);
+        if (!k_ok) {
+            a = mbf16x8_t{0, 0, 0, 0, 0, 0, 0, 0};
+#pragma unroll
+            for (int j = 0; j < 4; ++j) b[j] = a;
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b[j], acc[j], 0, 0, 0);
+    }
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int p = rows[tile * MOE_TILE + wave * 16 + 4 * g + i];
+        if (p < 0) continue;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int c = c0 + 16 * j + r;
+            if (c < H) y[(long)p * H + c] = f32_to_bf16(acc[j][i]);
+        }
+    }
+}
+
+template <typename ST>
+__global__ __launch_bounds__(256) void moe_combine_kernel(const bf16_t* __restrict__ y, const float* __restrict__ w,
+                                                          const ST* __restrict__ shared, int shared_parts,
+                                                          long shared_stride, const float* __restrict__ sg,
+                                                          float* __restrict__ out, long total, int H, int top) {
+    for (long i = (long)blockIdx.x * 256 + threadIdx.x; i < total; i += (long)gridDim.x * 256) {
+        const long t = i / H;
+        const int c = (int)(i - t * H);
+        float s = 0.f;
+        for (int k = 0; k < top; ++k) s += w[t * top + k] * to_f32(y[(t * top + k) * H + c]);
+        if (shared) {
+            float v = 0.f;
+            for (int p = 0; p < shared_parts; ++p) v += to_f32(shared[(long)p * shared_stride + i]);
+            s += (sg ? sg[t] : 1.0f) * v;
+        }
+        out[i] = s;
+    }
+}
+
+// scratch: rows int [max_tiles * 64], tile_expert int [max_tiles], n_tiles int [1], y bf16 [n * top, H];
+// max_tiles = ceil(n * top / 64) + E
+extern "C" const char* cpmcu_moe_experts_mfma(const void* h, long ldh, const void* wgu, const void* wd, const int* idx,
+                                              const float* w, const void* shared, int shared_dtype, int shared_parts,
+                                              long shared_stride, const float* sg, void* act, void* y, int* rows,
+                                              int* tile_expert, int* n_tiles, int max_tiles, float* out, int n, int H,
+                                              int F, int E, int top, hipStream_t stream) {
+    CPMCU_REQUIRE(n > 0 && H > 0 && F > 0 && E > 0 && top > 0, "moe_experts_mfma: empty shape");
+    CPMCU_REQUIRE(E <= MOE_MAX_EXPERTS, "moe_experts_mfma: %d experts (up to %d are taken)", E, MOE_MAX_EXPERTS);
+    CPMCU_REQUIRE(H % 8 == 0 && F % 8 == 0 && ldh % 8 == 0 && (uintptr_t)h % 16 == 0 && (uintptr_t)wgu % 16 == 0 &&
+                  (uintptr_t)wd % 16 == 0 && (uintptr_t)act % 16 == 0,
+                  "moe_experts_mfma: widths must be multiples of 8 and operands start on 16-byte borders (H=%d, F=%d)", H, F);
+    const long pairs = (long)n * top;
+    CPMCU_REQUIRE(max_tiles >= (pairs + MOE_TILE - 1) / MOE_TILE + E && max_tiles <= 65535,
+                  "moe_experts_mfma: %d tiles of scratch for %ld pairs of %d experts (at most 65535)", max_tiles, pairs, E);
+    moe_group_kernel<<<1, 1024, 0, stream>>>(idx, (int)pairs, E, rows, tile_expert, n_tiles, max_tiles);
+    CPMCU_LAUNCH_CHECK("moe_group");
+    moe_gated_mfma_kernel<<<dim3((F + 31) / 32, max_tiles), 256, 0, stream>>>((const bf16_t*)h, ldh, (const bf16_t*)wgu, rows,
+                                                                            tile_expert, n_tiles, (bf16_t*)act, H, F, top);
+    CPMCU_LAUNCH_CHECK("moe_gated_mfma");
+    moe_down_mfma_kernel<<<dim3((H + 63) / 64, max_tiles), 256, 0, stream>>>((const bf16_t*)act, (const bf16_t*)wd, rows,
+                                                                           tile_expert, n_tiles, (bf16_t*)y, H, F);
+    CPMCU_LAUNCH_CHECK("moe_down_mfma");
+    const long total = (long)n * H;
+    const int blocks = (int)((total + 255) / 256 < 8192 ? (total + 255) / 256 : 8192);
+    if (!shared || shared_dtype == CPMCU_F32)
+        moe_combine_kernel<float><<<blocks, 256, 0, stream>>>((const bf16_t*)y, w, (const float*)shared, shared_parts,
+                                                              shared_stride, sg, out, total, H, top);
+    else
+        moe_combine_kernel<bf16_t><<<blocks, 256, 0, stream>>>((const bf16_t*)y, w, (const bf16_t*)shared, shared_parts,
+                                                               shared_stride, sg, out, total, H, top);
+    CPMCU_LAUNCH_CHECK("moe_combine");
+    return nullptr;
+}

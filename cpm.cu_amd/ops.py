@@ -827,6 +827,54 @@ def moe_down(act: torch.Tensor, down: torch.Tensor, idx: torch.Tensor, weights: 
                                         _p(shared_gate), _p(out), c_int(n), c_int(H), c_int(F), c_int(top), _stream()))
 
 
+MOE_TILE = 64
+
+
+def moe_tiles(n: int, top: int, experts: int) -> int:
+    """Tiles of MOE_TILE rows that moe_experts_mfma's scratch must hold for n tokens: every expert's pairs fill whole
+    tiles, so up to one tile an expert is partly empty."""
+    return -(-(n * top) // MOE_TILE) + experts
+
+
+def moe_experts_mfma_ok(h: torch.Tensor, expert_size: int, n_tiles: int) -> bool:
+    return (h.dtype == torch.bfloat16 and h.shape[1] % 8 == 0 and expert_size % 8 == 0 and n_tiles <= 65535
+            and h.stride(0) % 8 == 0)
+
+
+def moe_experts_mfma(h: torch.Tensor, gate_up: torch.Tensor, down: torch.Tensor, idx: torch.Tensor, weights: torch.Tensor,
+                     out: torch.Tensor, act: torch.Tensor, y: torch.Tensor, rows: torch.Tensor, tile_expert: torch.Tensor,
+                     n_tiles: torch.Tensor, shared: Optional[torch.Tensor] = None,
+                     shared_gate: Optional[torch.Tensor] = None):
+    """moe_gated + moe_down for steps of many tokens, bf16 on the matrix cores: the (token, expert) pairs are grouped
+    by expert into tiles of MOE_TILE rows.  Scratch: act bf16 [n, top, F], y bf16 [n, top, H], rows int32
+    [tiles * MOE_TILE], tile_expert int32 [tiles], n_tiles int32 [1], tiles >= moe_tiles(n, top, E)."""
+    ldh = _ld(h, "experts input")
+    n, H = h.shape
+    _need(gate_up, "experts gate/up", torch.bfloat16, (None, None, H))
+    E, F = gate_up.shape[0], gate_up.shape[1] // 2
+    _need(down, "experts down", torch.bfloat16, (E, H, F))
+    _need(idx, "chosen experts", torch.int32, (n, None))
+    top = idx.shape[1]
+    _need(weights, "expert weights", torch.float32, (n, top))
+    _need(out, "experts out", torch.float32, (n, H))
+    _need(act, "experts act", torch.bfloat16, (n, top, F))
+    _need(y, "experts pair outputs", torch.bfloat16, (n, top, H))
+    _need(tile_expert, "experts tile map", torch.int32, (None,))
+    tiles = tile_expert.shape[0]
+    _need(rows, "experts tile rows", torch.int32, (tiles * MOE_TILE,))
+    _need(n_tiles, "experts tile count", torch.int32, (1,))
+    if h.dtype != torch.bfloat16:
+        raise KernelError("moe_experts_mfma: bfloat16 only")
+    sp, sstr = _parts_of(shared, n, H, "shared expert") if shared is not None else (0, 0)
+    if shared_gate is not None:
+        _need(shared_gate, "shared gate", torch.float32, (n,))
+    _check(_fn("moe", "cpmcu_moe_experts_mfma")(
+        _p(h), c_long(ldh), _p(gate_up), _p(down), _p(idx), _p(weights), _p(shared),
+        c_int(_code(shared) if shared is not None else 0), c_int(sp), c_long(sstr), _p(shared_gate), _p(act), _p(y),
+        _p(rows), _p(tile_expert), _p(n_tiles), c_int(tiles), _p(out), c_int(n), c_int(H), c_int(F), c_int(E), c_int(top),
+        _stream()))
+
+
 def latent_store(proj: torch.Tensor, q_out: torch.Tensor, nh: int, dim: int, rot: int, rank: int,
                  norm_w: Optional[torch.Tensor], eps: float, positions: torch.Tensor, tok_slot: torch.Tensor,
                  inv_freq: Optional[torch.Tensor], mag: float, kpool: Optional[torch.Tensor],

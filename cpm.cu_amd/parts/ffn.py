@@ -151,7 +151,18 @@ class RoutedExpertsFFN(FeedForward):
         shared = self.shared.forward(h, ctx) if self.shared is not None else None
         act = ctx.ws.get("moe.act", (n, self.top, self.expert_size), self.rt.dtype)
         out = ctx.ws.get("moe.out", (n, self.hidden_size), torch.float32)
+        tiles = ops.moe_tiles(n, self.top, self.experts)
         with ctx.timed("moe_experts"):
-            ops.moe_gated(h, self.gate_up, idx, act)
-            ops.moe_down(act, self.down, idx, wts, out, shared, sg)
+            if n > ops.SKINNY_MAX_ROWS and ops.moe_experts_mfma_ok(h, self.expert_size, tiles):
+                # many tokens: experts are shared by many of them; pairs grouped by expert, on the matrix cores
+                y = ctx.ws.get("moe.pair_out", (n, self.top, self.hidden_size), torch.bfloat16)
+                rows = ctx.ws.get("moe.tile_rows", (tiles * ops.MOE_TILE,), torch.int32)
+                tile_expert = ctx.ws.get("moe.tile_expert", (tiles,), torch.int32)
+                n_tiles = ctx.ws.get("moe.n_tiles", (1,), torch.int32)
+                ops.moe_experts_mfma(h, self.gate_up, self.down, idx, wts, out, act, y, rows, tile_expert, n_tiles,
+                                     shared, sg)
+            else:
+                # few tokens: an expert's weights stream once for every token that chose it
+                ops.moe_gated(h, self.gate_up, idx, act)
+                ops.moe_down(act, self.down, idx, wts, out, shared, sg)
         return out

@@ -355,6 +355,50 @@ def test_experts(dtype, shape):
     close(out2, want - sgate.double()[:, None] * shared.double().sum(0), "float32" if dtype == "float32" else "bfloat16")
 
 
+@pytest.mark.parametrize("shape", [(96, 40, 8, 3, 300), (104, 24, 6, 2, 65), (64, 24, 5, 1, 700), (128, 64, 16, 4, 1000),
+                                   (256, 136, 40, 6, 129)])
+def test_experts_of_many_tokens_on_the_matrix_cores(shape):
+    """Pairs grouped by expert in tiles of 64 rows: equal to the few-token kernels pair by pair, whatever row of a
+    tile a pair lands in; experts that nobody chose, experts with more than a tile of tokens, a last tile partly
+    empty."""
+    from cpmcu_amd import ops
+    Hd, F, E, top, n = shape
+    torch.manual_seed(44)
+    h = torch.randn(n, Hd).to(torch.bfloat16)
+    gu = (torch.randn(E, 2 * F, Hd) * 0.2).to(torch.bfloat16)
+    dn = (torch.randn(E, Hd, F) * 0.2).to(torch.bfloat16)
+    busy = max(E - 2, top)                                        # the last experts stay without tokens
+    idx = torch.stack([torch.randperm(busy)[:top] for _ in range(n)]).to(torch.int32)
+    idx[:n // 2, 0] = 0                                           # and the first is crowded
+    for t in range(n // 2):
+        if (idx[t, 1:] == 0).any():
+            idx[t, 1:][idx[t, 1:] == 0] = busy - 1 if busy - 1 not in idx[t].tolist() else idx[t, 0]
+    idx = torch.stack([torch.tensor(sorted(set(r.tolist())) + [e for e in range(busy) if e not in r.tolist()])[:top]
+                       for r in idx]).to(torch.int32)
+    w = torch.rand(n, top)
+    shared = torch.randn(n, Hd).to(torch.bfloat16)
+    sgate = torch.rand(n)
+    hd, gud, dnd, idxd, wd = dev(h), dev(gu), dev(dn), dev(idx), dev(w)
+    act = torch.empty(n, top, F, dtype=torch.bfloat16, device=DEV)
+    want = torch.empty(n, Hd, device=DEV)
+    ops.moe_gated(hd, gud, idxd, act)
+    ops.moe_down(act, gud.new_empty(0) if False else dnd, idxd, wd, want, dev(shared), dev(sgate))
+    tiles = ops.moe_tiles(n, top, E)
+    act2 = torch.empty_like(act)
+    y = torch.empty(n, top, Hd, dtype=torch.bfloat16, device=DEV)
+    rows = torch.empty(tiles * ops.MOE_TILE, dtype=torch.int32, device=DEV)
+    te, nt = torch.empty(tiles, dtype=torch.int32, device=DEV), torch.empty(1, dtype=torch.int32, device=DEV)
+    out = torch.empty(n, Hd, device=DEV)
+    for _ in range(2):
+        ops.moe_experts_mfma(hd, gud, dnd, idxd, wd, out, act2, y, rows, te, nt, dev(shared), dev(sgate))
+        close(act2, act.float().cpu(), "bfloat16")
+        close(out, want.cpu(), "bfloat16")
+    counts = torch.bincount(idx.flatten().long(), minlength=E)
+    assert int(nt) == int(((counts + 63) // 64).sum())
+    placed = rows[:int(nt) * 64].cpu()
+    assert sorted(placed[placed >= 0].tolist()) == list(range(n * top))
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_gates_of_a_parallel_layer(dtype):
     from cpmcu_amd import ops
