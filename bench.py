@@ -172,12 +172,14 @@ def main():
     ap.add_argument("--perf", action="store_true",
                     help="after the timed runs, a few eager steps with the engine's timers on: average ms by kernel "
                          "class (products / attention / selection / norms / head) on stderr and under 'timers'")
-    ap.add_argument("--scenario", default="headline", choices=["headline", "small_batch64", "sparse32k", "duvulix"],
+    ap.add_argument("--scenario", default="headline", choices=["headline", "small_batch64", "sparse32k", "duvulix", "gumodra"],
                     help="headline: the 8B shape at batch 8, context 4,096 (the default line); "
                          "small_batch64: the 0.5B shape, 64 unequal prompts through the generation loop; sparse32k: "
                          "the 8B shape with InfLLM-v2 at 32k context; duvulix: four Duvulix layers of a real model's "
                          "sizes (latent attention, chunked attention, Mamba-2, a layer that reads the first one's "
-                         "latent cache) beside four MiniCPM4-8B layers of equal width: decode and prefill of both")
+                         "latent cache) beside four MiniCPM4-8B layers of equal width: decode and prefill of both; gumodra: "
+                         "four Gumodra layers of a real model's sizes (windowed attention with a sink, mLSTM, dense and "
+                         "routed feed-forwards) beside the four Duvulix layers")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py: this engine runs on one GPU; --gpus {args.gpus} is not supported (no multi-GPU path exists)")
@@ -410,9 +412,89 @@ def duvulix_step_bytes(raw, esize, batch, context):
     return weights * esize + batch * per_seq, weights
 
 
+def config_gumodra():
+    """Four layers of sizes that resemble a real model's: width 4,096; attention with 32 heads on 8 kv heads of 128
+    (the keys double as values), 64 rotated features, a window of 2,048 tokens that keeps the first 128, a sink a
+    head; an mLSTM of 8 heads with keys of 256 and values of 512; SiLU-gated feed-forwards of 11,008; mixtures of 64
+    experts of 1,408 in 8 groups (4 kept), 6 a token, with a shared expert of 2,816."""
+    attn = {"heads": 32, "kv_heads": 8, "dim": 128, "vdim": 128, "scale": 128 ** -0.5,
+            "rot": {"base": 500000.0, "dims": 64}, "mask": {"size": 2048, "keep_first": 128}}
+    dense = {"kind": "dense", "ff": 11008}
+    moe = {"kind": "moe", "expert": {"ff": 1408}, "router": {"experts": 64, "top": 6, "groups": {"count": 8, "keep": 4}},
+           "shared": {"ff": 2816}}
+    return {
+        "architecture": "Gumodra", "vocab": 73448, "width": 4096, "norm": {"eps": 1e-6}, "embedding": {"scale": 12.0},
+        "layers": [
+            {"type": "attention", "mixer": dict(attn), "mlp": dense},
+            {"type": "attention", "mixer": dict(attn), "mlp": moe},
+            {"type": "mlstm", "mixer": {"heads": 8, "dim": 256, "vdim": 512, "gate_cap": 15.0}, "mlp": dense},
+            {"type": "attention", "mixer": dict(attn), "mlp": moe},
+        ],
+    }
+
+
+def gumodra_step_bytes(raw, esize, batch, context):
+    """Bytes a decode step must move: every matrix that the step reads once (of a mixture: the router, the shared
+    expert, and an expert for every (token, choice) pair, at most all of them), and per sequence what its mixers
+    read: keys and values of the window and of the kept first tokens, the recurrent state read and written."""
+    W = raw["width"]
+    weights = raw["vocab"] * W
+    per_seq = 0
+    for layer in raw["layers"]:
+        m = layer["mixer"]
+        if layer["type"] == "attention":
+            weights += (2 * m["heads"] * m["dim"] + m["kv_heads"] * m["dim"]) * W
+            mask = m.get("mask")
+            seen = context if not mask else min(context, mask["size"] + mask.get("keep_first", 0))
+            per_seq += seen * m["kv_heads"] * 2 * m["dim"] * esize
+        else:
+            hk, hv = m["heads"] * m["dim"], m["heads"] * m["vdim"]
+            weights += (2 * hk + 3 * hv + 2 * m["heads"]) * W
+            per_seq += 2 * 4 * (m["heads"] * m["dim"] * m["vdim"] + hk + m["heads"])
+        mlp = layer.get("mlp")
+        weights += W * W * (2 if mlp else 1)                       # the gates of the two results
+        if mlp and mlp["kind"] == "dense":
+            weights += 3 * mlp["ff"] * W
+        elif mlp:
+            r = mlp["router"]
+            weights += r["experts"] * W + (3 * mlp["shared"]["ff"] * W + W if mlp.get("shared") else 0)
+            weights += min(max(batch, 1) * r["top"], r["experts"]) * 3 * mlp["expert"]["ff"] * W
+    return weights * esize + batch * per_seq, weights
+
+
+def gumodra_prefill_params(raw):
+    """Matrix elements a prompt token is multiplied with (of a mixture: the chosen experts only)."""
+    W = raw["width"]
+    total = raw["vocab"] * W
+    for layer in raw["layers"]:
+        m = layer["mixer"]
+        if layer["type"] == "attention":
+            total += (2 * m["heads"] * m["dim"] + m["kv_heads"] * m["dim"]) * W
+        else:
+            total += (2 * m["heads"] * m["dim"] + 3 * m["heads"] * m["vdim"] + 2 * m["heads"]) * W
+        mlp = layer.get("mlp")
+        total += W * W * (2 if mlp else 1)
+        if mlp and mlp["kind"] == "dense":
+            total += 3 * mlp["ff"] * W
+        elif mlp:
+            total += mlp["router"]["experts"] * W + (3 * mlp["shared"]["ff"] * W if mlp.get("shared") else 0)
+            total += mlp["router"]["top"] * 3 * mlp["expert"]["ff"] * W
+    return total
+
+
 def duvulix_scenario(args, dev):
     """Decode and prefill of the Duvulix layer shapes beside the MiniCPM4-8B layer shape (equal width, equal
     number of layers, random weights): one JSON line with both models' figures and their timers by kernel class."""
+    layer_shapes_scenario(args, dev, "duvulix", "Duvulix", config_duvulix(), ("minicpm", config_8b(4)))
+
+
+def gumodra_scenario(args, dev):
+    """The same for the Gumodra layer shapes beside the Duvulix layer shapes (the package's other design of mixed
+    attention and recurrent layers; equal width, vocabulary and number of layers)."""
+    layer_shapes_scenario(args, dev, "gumodra", "Gumodra", config_gumodra(), ("duvulix", config_duvulix()))
+
+
+def layer_shapes_scenario(args, dev, first, title, first_raw, other):
     import torch
     import cpmcu_amd
     from cpmcu_amd import Engine, EngineOptions, StepEntry, ops
@@ -425,7 +507,7 @@ def duvulix_scenario(args, dev):
     next_tok = torch.zeros(64, dtype=torch.int32, device=dev)
     read_gbs = calibrate_read(dev)
     out = {}
-    for name, raw in (("duvulix", config_duvulix()), ("minicpm", config_8b(4))):
+    for name, raw in ((first, first_raw), other):
         arch = cpmcu_amd.get_architecture(raw.get("architecture") or raw["architectures"][0])
         cfg = arch.config_class.from_dict(raw)
         per_seq = -(-(args.context + args.steps + args.warmup + 64) // 64) * 64
@@ -475,9 +557,14 @@ def duvulix_scenario(args, dev):
                 best = dt if best is None else min(best, dt)
             return best
 
+        prefill_params = None
         if name == "duvulix":
             step_bytes = lambda b: duvulix_step_bytes(raw, esize, b, args.context)[0]
             params = duvulix_step_bytes(raw, esize, 0, 0)[1]
+        elif name == "gumodra":
+            step_bytes = lambda b: gumodra_step_bytes(raw, esize, b, args.context)[0]
+            params = gumodra_step_bytes(raw, esize, args.batch, 0)[1]
+            prefill_params = gumodra_prefill_params(raw)
         else:
             step_bytes = lambda b: weight_bytes_per_step(cfg, esize) + b * args.context * kv_bytes_per_token(cfg, esize)
             params = weight_bytes_per_step(cfg, esize) // esize
@@ -492,7 +579,7 @@ def duvulix_scenario(args, dev):
             print(f"[bench] {name}: decode batch {b} context {args.context}: {ms:.3f} ms a step, {gbs:.0f} GB/s", file=sys.stderr, flush=True)
         if not args.no_prefill:
             dt = prefill()
-            flops = 2.0 * params * n_prefill
+            flops = 2.0 * (prefill_params or params) * n_prefill
             rec["prefill"] = {"tokens": n_prefill, "ms": round(dt * 1e3, 3), "tokens_per_s": round(n_prefill / dt, 1),
                               "matrix_flops_frac_of_peak": round(flops / dt / PEAK_FLOPS["bf16" if esize == 2 else "fp32"], 4)}
             print(f"[bench] {name}: prefill of {n_prefill} tokens: {dt * 1e3:.2f} ms", file=sys.stderr, flush=True)
@@ -514,15 +601,15 @@ def duvulix_scenario(args, dev):
         out[name] = rec
         del eng
         torch.cuda.empty_cache()
-    d = out["duvulix"]["decode"][str(args.batch)]
+    d = out[first]["decode"][str(args.batch)]
     print(json.dumps({
-        "metric": f"Duvulix layer shapes (4 layers, width 4096): decode tok/s at batch {args.batch}, context {args.context}",
+        "metric": f"{title} layer shapes (4 layers, width 4096): decode tok/s at batch {args.batch}, context {args.context}",
         "value": d["tokens_per_s"], "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": d["ms_per_step"], "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16" if esize == 2 else "fp32", "data": "synthetic",
-        "config": {"model": "Duvulix layer shapes beside MiniCPM4-8B layer shapes, 4 layers each, random weights",
+        "config": {"model": f"{title} layer shapes beside {other[0]} layer shapes, 4 layers each, random weights",
                    "global_batch": args.batch, "seq_len": args.context, "parallelism": "1gpu",
-                   "hip_graph": bool(args.hip_graph), "duvulix": config_duvulix()},
+                   "hip_graph": bool(args.hip_graph), first: first_raw},
         "read_kernel_gbs": round(read_gbs, 1), "models": out}))
 
 
@@ -530,6 +617,9 @@ def other_scenarios(args, dev):
     """The further workloads, each one JSON line of the same shape."""
     if args.scenario == "duvulix":
         duvulix_scenario(args, dev)
+        return
+    if args.scenario == "gumodra":
+        gumodra_scenario(args, dev)
         return
     import torch
     from cpmcu_amd import Engine, EngineOptions, StepEntry

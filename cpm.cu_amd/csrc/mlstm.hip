@@ -8,50 +8,61 @@
 //   y_t = S_t^T q_t / (max(|n_t . q_t|, exp(-m_t)) + 1e-6)
 //
 // q, k, v and the raw gates i, f are columns of one projection (q is multiplied by `q_scale` as it is read);
-// gates, decays, the state and the output are float.  S, n and m live per cache slot and are carried from step to
+// gates, decays, the state and the output are float.  The kernel leaves S_t^T q_t and the denominator side by side;
+// the head norm that follows divides.  S, n and m live per cache slot and are carried from step to
 // step, so a step of any number of tokens continues where the last one ended.
 #include "common.h"
 
-#define ML_PB 32        // value columns a workgroup
-#define ML_L 8          // lanes a column: key index c = l + 8 i
+// A workgroup of 256 threads walks ML_PB = 256 / ML_L columns; a column's d state values lie over ML_L neighbouring
+// lanes (8 or 16: key index c = l + ML_L i), which sum their shares inside the vector unit.  Keys beyond 128
+// features take 16 lanes a column: twice the workgroups, and half the chain of dependent additions a token.
 
 __device__ inline float log_sigmoid_f(float v) { return fminf(v, 0.f) - log1pf(expf(-fabsf(v))); }
 
-// grid (sequences, heads, ceil(dv / 32)), 256 threads.  proj: [n, ld]; q at column q_off + h * d, k at k_off + h * d,
-// v at v_off + h * dv, raw gates at i_off + h and f_off + h.  S: [slots][heads][dv][d], nst: [slots][heads][d],
-// mst: [slots][heads]; y: float [n, heads * dv].
-template <int NR, int ML_TT, typename T>   // ML_TT: tokens a tile in LDS
+// grid (sequences, heads, ceil((dv + 1) / ML_PB)), 256 threads.  proj: [n, ld]; q at column q_off + h * d, k at
+// k_off + h * d, v at v_off + h * dv, raw gates at i_off + h and f_off + h.  S: [slots][heads][dv][d],
+// nst: [slots][heads][d], mst: [slots][heads].
+//
+// The normaliser n obeys the recurrence of a column of S whose value is always 1, so it is walked as column dv:
+// columns 0 .. dv - 1 give the unnormalised y = S^T q (float [n, heads * dv]) and column dv gives n . q, from which
+// den[t, h] = max(|n . q|, exp(-m)) + 1e-6 (float [n, heads]); whoever reads y divides by den (the head norm does).
+// Tiles of ML_TT tokens pass through LDS; the running maximum of a tile is walked by one thread first (additions and
+// maxima only), then the tile's exponentials are formed side by side, so the walk over the state itself holds
+// nothing but multiply-adds.
+template <int NR, int ML_L, int ML_TT, typename T>
 __global__ __launch_bounds__(256) void mlstm_scan_kernel(const T* __restrict__ proj, long ld, long q_off, long k_off,
                                                          long v_off, long i_off, long f_off,
                                                          const float* __restrict__ i_bias,
                                                          const float* __restrict__ f_bias, float cap, float q_scale,
                                                          float* __restrict__ S_state, float* __restrict__ n_state,
                                                          float* __restrict__ m_state, float* __restrict__ y,
-                                                         const int* __restrict__ cu_q, const int* __restrict__ seq_slot,
-                                                         int heads, int d, int dv, int write_state) {
+                                                         float* __restrict__ den, const int* __restrict__ cu_q,
+                                                         const int* __restrict__ seq_slot, int heads, int d, int dv,
+                                                         int write_state) {
+    constexpr int ML_PB = 256 / ML_L;               // columns a workgroup
     constexpr int NS = NR * ML_L;                   // key features, padded
     constexpr int QK = ML_TT * NS / 256;            // q (and k) values a thread brings a tile
     constexpr int XV = ML_TT * ML_PB / 256;         // v values a thread brings a tile
     __shared__ float qs[ML_TT][NS];
     __shared__ float ks[ML_TT][NS];
     __shared__ float vs[ML_TT][ML_PB];
-    __shared__ float as_[ML_TT], bs_[ML_TT];
+    __shared__ float keep_s[ML_TT], take_s[ML_TT], em_s[ML_TT];
+    __shared__ float m_carry;
     const int b = blockIdx.x, h = blockIdx.y, p0 = blockIdx.z * ML_PB;
     const int start = cu_q[b], q = cu_q[b + 1] - start;
     const int slot = seq_slot[b];
     const int pl = threadIdx.x / ML_L, l = threadIdx.x % ML_L;
     const int p = p0 + pl;
-    const bool p_ok = p < dv;
-    float S[NR], nv[NR];
-    float* sp = S_state + (((long)slot * heads + h) * dv + (p_ok ? p : 0)) * d;
-    float* np = n_state + ((long)slot * heads + h) * d;
+    const bool p_ok = p <= dv, is_n = p == dv;
+    float S[NR];
+    float* sp = is_n ? n_state + ((long)slot * heads + h) * d
+                     : S_state + (((long)slot * heads + h) * dv + (p_ok ? p : 0)) * d;
 #pragma unroll
     for (int i = 0; i < NR; ++i) {
         const int c = l + ML_L * i;
         S[i] = (p_ok && c < d) ? sp[c] : 0.f;
-        nv[i] = c < d ? np[c] : 0.f;
     }
-    float m = m_state[(long)slot * heads + h];
+    if (threadIdx.x == 0) m_carry = m_state[(long)slot * heads + h];
     const float bi = i_bias[h], bf = f_bias[h], inv_cap = 1.0f / cap;
     float rq[QK], rk[QK], rx[XV], ri = 0.f, rf = 0.f;
     auto fetch = [&](int t0) {
@@ -68,8 +79,10 @@ __global__ __launch_bounds__(256) void mlstm_scan_kernel(const T* __restrict__ p
 #pragma unroll
         for (int e2 = 0; e2 < XV; ++e2) {
             const int e = threadIdx.x + e2 * 256;
-            const int tt = e / ML_PB, pp = e % ML_PB;
-            rx[e2] = (tt < tn && p0 + pp < dv) ? to_f32(proj[(long)(start + t0 + tt) * ld + v_off + (long)h * dv + p0 + pp]) : 0.f;
+            const int tt = e / ML_PB, pp = p0 + e % ML_PB;
+            const long at = (long)(start + t0 + min(tt, tn - 1)) * ld + v_off + (long)h * dv + min(pp, dv - 1);
+            const float v = to_f32(proj[at]);
+            rx[e2] = tt < tn ? (pp < dv ? v : (pp == dv ? 1.0f : 0.f)) : 0.f;
         }
         if ((int)threadIdx.x < tn) {
             const T* row = proj + (long)(start + t0 + threadIdx.x) * ld + h;
@@ -92,57 +105,77 @@ __global__ __launch_bounds__(256) void mlstm_scan_kernel(const T* __restrict__ p
             const int e = threadIdx.x + e2 * 256;
             vs[e / ML_PB][e % ML_PB] = rx[e2];
         }
+        if ((int)threadIdx.x < tn) {                 // log gates, parked where their exponentials will stand
+            take_s[threadIdx.x] = cap * tanhf((ri + bi) * inv_cap);
+            keep_s[threadIdx.x] = log_sigmoid_f(cap * tanhf((rf + bf) * inv_cap));
+        }
+        __syncthreads();
+        if (threadIdx.x == 0) {                      // the running maximum through the tile, in registers
+            float av[ML_TT], bv[ML_TT];
+#pragma unroll
+            for (int tt = 0; tt < ML_TT; ++tt) {
+                av[tt] = take_s[tt];
+                bv[tt] = keep_s[tt];
+            }
+            float m = m_carry;
+#pragma unroll
+            for (int tt = 0; tt < ML_TT; ++tt) {
+                const float m_new = tt < tn ? fmaxf(bv[tt] + m, av[tt]) : m;
+                bv[tt] = bv[tt] + m - m_new;
+                av[tt] = av[tt] - m_new;
+                m = m_new;
+                keep_s[tt] = bv[tt];
+                take_s[tt] = av[tt];
+                em_s[tt] = -m_new;
+            }
+            m_carry = m;
+        }
+        __syncthreads();
         if ((int)threadIdx.x < tn) {
-            as_[threadIdx.x] = cap * tanhf((ri + bi) * inv_cap);
-            bs_[threadIdx.x] = log_sigmoid_f(cap * tanhf((rf + bf) * inv_cap));
+            keep_s[threadIdx.x] = expf(keep_s[threadIdx.x]);
+            take_s[threadIdx.x] = expf(take_s[threadIdx.x]);
+            em_s[threadIdx.x] = expf(em_s[threadIdx.x]);
         }
         __syncthreads();
         if (t0 + ML_TT < q) fetch(t0 + ML_TT);
         for (int tt = 0; tt < tn; ++tt) {
-            const float a = as_[tt], bb = bs_[tt];
-            const float m_new = fmaxf(bb + m, a);
-            const float keep = expf(bb + m - m_new), take = expf(a - m_new);
-            m = m_new;
-            const float tv = take * vs[tt][pl];
-            float num = 0.f, dot = 0.f;
+            const float keep = keep_s[tt];
+            const float tv = take_s[tt] * vs[tt][pl];
+            float part[4] = {0.f, 0.f, 0.f, 0.f};       // four chains of additions side by side
 #pragma unroll
             for (int i = 0; i < NR; ++i) {
                 const int c = l + ML_L * i;
-                const float kk = ks[tt][c], qq = qs[tt][c];
-                S[i] = keep * S[i] + tv * kk;
-                nv[i] = keep * nv[i] + take * kk;
-                num += S[i] * qq;
-                dot += nv[i] * qq;
+                S[i] = keep * S[i] + tv * ks[tt][c];
+                part[i & 3] += S[i] * qs[tt][c];
             }
-            // the column's 8 lanes are neighbours: sums inside the vector unit
+            float num = (part[0] + part[1]) + (part[2] + part[3]);
+            // the column's 8 lanes are neighbours: the sum inside the vector unit
             num += CPMCU_DPP(num, 0xB1);
             num += CPMCU_DPP(num, 0x4E);
             num += CPMCU_DPP(num, 0x141);
-            dot += CPMCU_DPP(dot, 0xB1);
-            dot += CPMCU_DPP(dot, 0x4E);
-            dot += CPMCU_DPP(dot, 0x141);
+            if (ML_L == 16) num += CPMCU_DPP(num, 0x140);
             if (l == 0 && p_ok) {
-                const float den = fmaxf(fabsf(dot), expf(-m)) + 1e-6f;
-                y[(long)(start + t0 + tt) * heads * dv + (long)h * dv + p] = num / den;
+                const long t = start + t0 + tt;
+                if (is_n) den[t * heads + h] = fmaxf(fabsf(num), em_s[tt]) + 1e-6f;
+                else y[t * heads * dv + (long)h * dv + p] = num;
             }
         }
     }
+    __syncthreads();
     if (write_state) {
 #pragma unroll
         for (int i = 0; i < NR; ++i) {
             const int c = l + ML_L * i;
             if (p_ok && c < d) sp[c] = S[i];
-            // every workgroup of a head walks the same n and m; the first one writes them
-            if (blockIdx.z == 0 && pl == 0 && c < d) np[c] = nv[i];
         }
-        if (blockIdx.z == 0 && threadIdx.x == 0) m_state[(long)slot * heads + h] = m;
+        if (blockIdx.z == 0 && threadIdx.x == 0) m_state[(long)slot * heads + h] = m_carry;
     }
 }
 
 extern "C" const char* cpmcu_mlstm_scan(const void* proj, long ld, int dtype, long q_off, long k_off, long v_off,
                                         long i_off, long f_off, const float* i_bias, const float* f_bias, float cap,
                                         float q_scale, float* S_state, float* n_state, float* m_state, float* y,
-                                        const int* cu_q, const int* seq_slot, int n_seqs, int heads, int d, int dv,
+                                        float* den, const int* cu_q, const int* seq_slot, int n_seqs, int heads, int d, int dv,
                                         int write_state, hipStream_t stream) {
     CPMCU_REQUIRE(n_seqs > 0 && heads > 0 && d > 0 && dv > 0, "mlstm_scan: empty shape");
     CPMCU_REQUIRE(d <= 256, "mlstm_scan: a key size of %d is not supported (at most 256)", d);
@@ -150,21 +183,23 @@ extern "C" const char* cpmcu_mlstm_scan(const void* proj, long ld, int dtype, lo
     CPMCU_REQUIRE(q_off >= 0 && k_off >= 0 && v_off >= 0 && i_off >= 0 && f_off >= 0 && q_off + (long)heads * d <= ld &&
                   k_off + (long)heads * d <= ld && v_off + (long)heads * dv <= ld && i_off + heads <= ld && f_off + heads <= ld,
                   "mlstm_scan: columns beyond rows of %ld", ld);
-    const int pb = (dv + ML_PB - 1) / ML_PB;
+    const int lanes = d > 128 ? 16 : 8, cols = 256 / lanes;
+    const int pb = (dv + 1 + cols - 1) / cols;       // the normaliser is walked as column dv
     CPMCU_REQUIRE(heads <= 65535 && pb <= 65535, "mlstm_scan: shape exceeds the launch grid");
     dim3 grid(n_seqs, heads, pb);
-    const int need = (d + ML_L - 1) / ML_L;
-#define LAUNCH(NRv, TTv, Tv)                                                                                             \
-    mlstm_scan_kernel<NRv, TTv, Tv><<<grid, 256, 0, stream>>>((const Tv*)proj, ld, q_off, k_off, v_off, i_off, f_off, i_bias, \
-                                                         f_bias, cap, q_scale, S_state, n_state, m_state, y, cu_q,  \
-                                                         seq_slot, heads, d, dv, write_state)
-#define BY_NR(Tv)                            \
-    do {                                     \
-        if (need <= 2) LAUNCH(2, 32, Tv);        \
-        else if (need <= 4) LAUNCH(4, 32, Tv);   \
-        else if (need <= 8) LAUNCH(8, 32, Tv);   \
-        else if (need <= 16) LAUNCH(16, 32, Tv); \
-        else LAUNCH(32, 16, Tv);                 \
+    const int need = (d + lanes - 1) / lanes;
+#define LAUNCH(NRv, Lv, TTv, Tv)                                                                                     \
+    mlstm_scan_kernel<NRv, Lv, TTv, Tv><<<grid, 256, 0, stream>>>((const Tv*)proj, ld, q_off, k_off, v_off, i_off,   \
+                                                                  f_off, i_bias, f_bias, cap, q_scale, S_state,      \
+                                                                  n_state, m_state, y, den, cu_q, seq_slot, heads,   \
+                                                                  d, dv, write_state)
+#define BY_NR(Tv)                                  \
+    do {                                           \
+        if (lanes == 16) LAUNCH(16, 16, 16, Tv);   \
+        else if (need <= 2) LAUNCH(2, 8, 32, Tv);  \
+        else if (need <= 4) LAUNCH(4, 8, 32, Tv);  \
+        else if (need <= 8) LAUNCH(8, 8, 32, Tv);  \
+        else LAUNCH(16, 8, 32, Tv);                \
     } while (0)
     if (dtype == CPMCU_F32) BY_NR(float);
     else if (dtype == CPMCU_BF16) BY_NR(bf16_t);

@@ -58,9 +58,9 @@ __device__ inline float lane_dot(const TA* __restrict__ a, const TB* __restrict_
 
 __device__ inline float wave_min_f(float v) { return -wave_max(-v); }
 
-// grid (tokens), 256 threads
+// grid (tokens), 256 or 1024 threads: the wavefronts share the experts' logits, the first one chooses
 template <typename T>
-__global__ __launch_bounds__(256) void moe_route_kernel(const T* __restrict__ h, long ldh, const float* __restrict__ wr,
+__global__ __launch_bounds__(1024) void moe_route_kernel(const T* __restrict__ h, long ldh, const float* __restrict__ wr,
                                                         const float* __restrict__ correction,
                                                         const float* __restrict__ w_sg, int H, int E, int n_groups,
                                                         int keep_groups, int top, int* __restrict__ idx_out,
@@ -72,7 +72,8 @@ __global__ __launch_bounds__(256) void moe_route_kernel(const T* __restrict__ h,
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
     const T* hr = h + t * ldh;
     const bool vec = (H % 8 == 0) && (ldh % 8 == 0) && ((uintptr_t)h % 32 == 0) && ((uintptr_t)wr % 32 == 0);
-    for (int e = wave; e < E + (w_sg ? 1 : 0); e += 4) {
+    const int n_waves = blockDim.x >> 6;
+    for (int e = wave; e < E + (w_sg ? 1 : 0); e += n_waves) {
         const float* row = e < E ? wr + (long)e * H : w_sg;
         const bool v = vec && (e < E || (uintptr_t)w_sg % 32 == 0);
         const float s = wave_sum(lane_dot<T, float>(hr, row, H, lane, v));
@@ -155,11 +156,12 @@ extern "C" const char* cpmcu_moe_route(const void* h, long ldh, int dtype, const
     CPMCU_REQUIRE(top >= 1 && top <= keep_groups * (E / n_groups), "moe_route: %d experts a token of %d that may be chosen",
                   top, keep_groups * (E / n_groups));
     CPMCU_REQUIRE(!w_sg || sg_out, "moe_route: a place for the shared gate is missing");
+    const int block = E + 1 > 16 ? 1024 : 256;
     if (dtype == CPMCU_F32)
-        moe_route_kernel<float><<<n, 256, 0, stream>>>((const float*)h, ldh, wr, correction, w_sg, H, E, n_groups,
+        moe_route_kernel<float><<<n, block, 0, stream>>>((const float*)h, ldh, wr, correction, w_sg, H, E, n_groups,
                                                        keep_groups, top, idx_out, w_out, sg_out);
     else if (dtype == CPMCU_BF16)
-        moe_route_kernel<bf16_t><<<n, 256, 0, stream>>>((const bf16_t*)h, ldh, wr, correction, w_sg, H, E, n_groups,
+        moe_route_kernel<bf16_t><<<n, block, 0, stream>>>((const bf16_t*)h, ldh, wr, correction, w_sg, H, E, n_groups,
                                                         keep_groups, top, idx_out, w_out, sg_out);
     else
         CPMCU_FAIL("moe_route: unknown dtype %d", dtype);
@@ -269,9 +271,10 @@ extern "C" const char* cpmcu_moe_down(const void* act, int dtype, const void* wd
 //  * moe_group_kernel (one workgroup): counts the pairs of every expert, gives every expert whole tiles of 64 rows
 //    (rows[tile * 64 + i] = pair, -1 in a tile's unused rows), tile_expert[tile] and the number of tiles.  Which row
 //    of its expert's tiles a pair gets depends on timing; its result does not (a row's sums are its own).
-//  * moe_gated_mfma_kernel: act[pair] = silu(Wg_e h_t) * (Wu_e h_t); a wavefront owns 16 rows of a tile and 32
-//    features (two tiles of gate rows, two of up rows), operands straight from memory.
-//  * moe_down_mfma_kernel: y[pair] = Wd_e act[pair] (bf16); a wavefront owns 16 rows and 64 columns.
+//  * moe_gated_mfma_kernel: act[pair] = silu(Wg_e h_t) * (Wu_e h_t); a wavefront owns the 64 rows of a tile and 32
+//    features (two tiles of gate rows, two of up rows): 16 matrix instructions for 8 operand loads, operands
+//    straight from memory (the 4 wavefronts of a workgroup read the same rows of h, which meet in the CU's cache).
+//  * moe_down_mfma_kernel: y[pair] = Wd_e act[pair] (bf16); a wavefront owns the 64 rows and 64 columns.
 //  * moe_combine_kernel: out[t] = sum_k w[t, k] y[t, k] (+ sg[t] * shared[t]) in float, k in order.
 // ===========================================================================
 typedef __bf16 mbf16x8_t __attribute__((ext_vector_type(8)));
@@ -308,7 +311,7 @@ __global__ __launch_bounds__(1024) void moe_group_kernel(const int* __restrict__
     }
 }
 
-// grid (ceil(F / 32), max_tiles), 256 threads
+// grid (ceil(F / 128), max_tiles), 256 threads: a wavefront takes all 64 rows of the tile and 32 features
 __global__ __launch_bounds__(256) void moe_gated_mfma_kernel(const bf16_t* __restrict__ h, long ldh,
                                                              const bf16_t* __restrict__ wgu, const int* __restrict__ rows,
                                                              const int* __restrict__ tile_expert,
@@ -319,53 +322,62 @@ __global__ __launch_bounds__(256) void moe_gated_mfma_kernel(const bf16_t* __res
     const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
     const int lane = threadIdx.x & 63, r = lane & 15, g = lane >> 4;
     const int e = tile_expert[tile];
-    const int f0 = blockIdx.x * 32;
-    const int pair = rows[tile * MOE_TILE + wave * 16 + r];
-    const bool row_ok = pair >= 0;
-    const bf16_t* xp = h + (long)(row_ok ? pair / top : 0) * ldh + g * 8;
-    const bf16_t* wp = wgu + (long)e * 2 * F * H + g * 8;
-    mfloatx4_t acc[4];
+    const int f0 = blockIdx.x * 128 + wave * 32;
+    if (f0 >= F) return;
+    const bf16_t* xp[4];
 #pragma unroll
-    for (int j = 0; j < 4; ++j) acc[j] = mfloatx4_t{0.f, 0.f, 0.f, 0.f};
+    for (int rt = 0; rt < 4; ++rt) {
+        const int pair = rows[tile * MOE_TILE + rt * 16 + r];
+        xp[rt] = h + (long)(pair >= 0 ? pair / top : 0) * ldh + g * 8;
+    }
+    const bf16_t* wp = wgu + (long)e * 2 * F * H + g * 8;
+    mfloatx4_t acc[4][4];
+#pragma unroll
+    for (int rt = 0; rt < 4; ++rt)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[rt][j] = mfloatx4_t{0.f, 0.f, 0.f, 0.f};
     long wrow[4];
 #pragma unroll
     for (int j = 0; j < 4; ++j) {                 // j = 0, 1: gate rows f0 + 16 j + r; j = 2, 3: their up rows
         const int f = min(f0 + 16 * (j & 1) + r, F - 1);
         wrow[j] = (long)((j >> 1) * F + f) * H;
     }
-#pragma unroll 2
     for (int k0 = 0; k0 < H; k0 += 32) {
         const bool k_ok = k0 + g * 8 < H;
         const int kk = k_ok ? k0 : k0 - g * 8;       // a lane beyond the row's end reads the step's first columns (in range) and is zeroed
-        mbf16x8_t a = *(const mbf16x8_t*)(xp + kk);
-        mbf16x8_t b[4];
+        mbf16x8_t a[4], b[4];
+#pragma unroll
+        for (int rt = 0; rt < 4; ++rt) a[rt] = *(const mbf16x8_t*)(xp[rt] + kk);
 #pragma unroll
         for (int j = 0; j < 4; ++j) b[j] = *(const mbf16x8_t*)(wp + wrow[j] + kk);
         if (!k_ok) {
-            a = mbf16x8_t{0, 0, 0, 0, 0, 0, 0, 0};
 #pragma unroll
-            for (int j = 0; j < 4; ++j) b[j] = a;
+            for (int j = 0; j < 4; ++j) a[j] = b[j] = mbf16x8_t{0, 0, 0, 0, 0, 0, 0, 0};
         }
 #pragma unroll
-        for (int j = 0; j < 4; ++j) acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b[j], acc[j], 0, 0, 0);
+        for (int rt = 0; rt < 4; ++rt)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) acc[rt][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[rt], b[j], acc[rt][j], 0, 0, 0);
     }
-    // lane (feature column r, g): acc[j][i] belongs to the tile's row wave * 16 + 4 g + i
+    // lane (feature column r, g): acc[rt][j][i] belongs to the tile's row rt * 16 + 4 g + i
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const int p = rows[tile * MOE_TILE + wave * 16 + 4 * g + i];
-        if (p < 0) continue;
+    for (int rt = 0; rt < 4; ++rt)
 #pragma unroll
-        for (int j = 0; j < 2; ++j) {
-            const int f = f0 + 16 * j + r;
-            if (f < F) {
-                const float gt = acc[j][i], up = acc[2 + j][i];
-                act[(long)p * F + f] = f32_to_bf16(gt / (1.0f + expf(-gt)) * up);
+        for (int i = 0; i < 4; ++i) {
+            const int p = rows[tile * MOE_TILE + rt * 16 + 4 * g + i];
+            if (p < 0) continue;
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                const int f = f0 + 16 * j + r;
+                if (f < F) {
+                    const float gt = acc[rt][j][i], up = acc[rt][2 + j][i];
+                    act[(long)p * F + f] = f32_to_bf16(gt / (1.0f + expf(-gt)) * up);
+                }
             }
         }
-    }
 }
 
-// grid (ceil(H / 64), max_tiles), 256 threads
+// grid (ceil(H / 256), max_tiles), 256 threads: a wavefront takes all 64 rows of the tile and 64 columns
 __global__ __launch_bounds__(256) void moe_down_mfma_kernel(const bf16_t* __restrict__ act, const bf16_t* __restrict__ wd,
                                                             const int* __restrict__ rows,
                                                             const int* __restrict__ tile_expert,
@@ -376,42 +388,52 @@ __global__ __launch_bounds__(256) void moe_down_mfma_kernel(const bf16_t* __rest
     const int wave = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 6));
     const int lane = threadIdx.x & 63, r = lane & 15, g = lane >> 4;
     const int e = tile_expert[tile];
-    const int c0 = blockIdx.x * 64;
-    const int pair = rows[tile * MOE_TILE + wave * 16 + r];
-    const bf16_t* xp = act + (long)(pair >= 0 ? pair : 0) * F + g * 8;
-    const bf16_t* wp = wd + (long)e * H * F + g * 8;
-    mfloatx4_t acc[4];
+    const int c0 = blockIdx.x * 256 + wave * 64;
+    if (c0 >= H) return;
+    const bf16_t* xp[4];
 #pragma unroll
-    for (int j = 0; j < 4; ++j) acc[j] = mfloatx4_t{0.f, 0.f, 0.f, 0.f};
+    for (int rt = 0; rt < 4; ++rt) {
+        const int pair = rows[tile * MOE_TILE + rt * 16 + r];
+        xp[rt] = act + (long)(pair >= 0 ? pair : 0) * F + g * 8;
+    }
+    const bf16_t* wp = wd + (long)e * H * F + g * 8;
+    mfloatx4_t acc[4][4];
+#pragma unroll
+    for (int rt = 0; rt < 4; ++rt)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) acc[rt][j] = mfloatx4_t{0.f, 0.f, 0.f, 0.f};
     long wrow[4];
 #pragma unroll
     for (int j = 0; j < 4; ++j) wrow[j] = (long)min(c0 + 16 * j + r, H - 1) * F;
-#pragma unroll 2
     for (int k0 = 0; k0 < F; k0 += 32) {
         const bool k_ok = k0 + g * 8 < F;
-        const int kk = k_ok ? k0 : k0 - g * 8;       // a lane beyond the row's end reads the step's first columns (in range) and is zeroed
-        mbf16x8_t a = *(const mbf16x8_t*)(xp + kk);
-        mbf16x8_t b[4];
+        const int kk = k_ok ? k0 : k0 - g * 8;
+        mbf16x8_t a[4], b[4];
+#pragma unroll
+        for (int rt = 0; rt < 4; ++rt) a[rt] = *(const mbf16x8_t*)(xp[rt] + kk);
 #pragma unroll
         for (int j = 0; j < 4; ++j) b[j] = *(const mbf16x8_t*)(wp + wrow[j] + kk);
         if (!k_ok) {
-            a = mbf16x8_t{0, 0, 0, 0, 0, 0, 0, 0};
 #pragma unroll
-            for (int j = 0; j < 4; ++j) b[j] = a;
+            for (int j = 0; j < 4; ++j) a[j] = b[j] = mbf16x8_t{0, 0, 0, 0, 0, 0, 0, 0};
         }
 #pragma unroll
-        for (int j = 0; j < 4; ++j) acc[j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b[j], acc[j], 0, 0, 0);
+        for (int rt = 0; rt < 4; ++rt)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) acc[rt][j] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[rt], b[j], acc[rt][j], 0, 0, 0);
     }
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        const int p = rows[tile * MOE_TILE + wave * 16 + 4 * g + i];
-        if (p < 0) continue;
+    for (int rt = 0; rt < 4; ++rt)
 #pragma unroll
-        for (int j = 0; j < 4; ++j) {
-            const int c = c0 + 16 * j + r;
-            if (c < H) y[(long)p * H + c] = f32_to_bf16(acc[j][i]);
+        for (int i = 0; i < 4; ++i) {
+            const int p = rows[tile * MOE_TILE + rt * 16 + 4 * g + i];
+            if (p < 0) continue;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int c = c0 + 16 * j + r;
+                if (c < H) y[(long)p * H + c] = f32_to_bf16(acc[rt][j][i]);
+            }
         }
-    }
 }
 
 template <typename ST>
@@ -450,10 +472,10 @@ extern "C" const char* cpmcu_moe_experts_mfma(const void* h, long ldh, const voi
                   "moe_experts_mfma: %d tiles of scratch for %ld pairs of %d experts (at most 65535)", max_tiles, pairs, E);
     moe_group_kernel<<<1, 1024, 0, stream>>>(idx, (int)pairs, E, rows, tile_expert, n_tiles, max_tiles);
     CPMCU_LAUNCH_CHECK("moe_group");
-    moe_gated_mfma_kernel<<<dim3((F + 31) / 32, max_tiles), 256, 0, stream>>>((const bf16_t*)h, ldh, (const bf16_t*)wgu, rows,
+    moe_gated_mfma_kernel<<<dim3((F + 127) / 128, max_tiles), 256, 0, stream>>>((const bf16_t*)h, ldh, (const bf16_t*)wgu, rows,
                                                                             tile_expert, n_tiles, (bf16_t*)act, H, F, top);
     CPMCU_LAUNCH_CHECK("moe_gated_mfma");
-    moe_down_mfma_kernel<<<dim3((H + 63) / 64, max_tiles), 256, 0, stream>>>((const bf16_t*)act, (const bf16_t*)wd, rows,
+    moe_down_mfma_kernel<<<dim3((H + 255) / 256, max_tiles), 256, 0, stream>>>((const bf16_t*)act, (const bf16_t*)wd, rows,
                                                                            tile_expert, n_tiles, (bf16_t*)y, H, F);
     CPMCU_LAUNCH_CHECK("moe_down_mfma");
     const long total = (long)n * H;

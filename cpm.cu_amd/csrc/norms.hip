@@ -28,16 +28,19 @@ template <typename XT, typename ZT, typename OT>
 __global__ __launch_bounds__(256) void rms_norm_groups_kernel(const XT* __restrict__ x, long ldx,
                                                               const ZT* __restrict__ z, long ldz,
                                                               const float* __restrict__ weight, OT* __restrict__ out,
-                                                              long ldo, int W, float eps, int gate_after) {
+                                                              long ldo, int W, float eps, int gate_after,
+                                                              const float* __restrict__ divisor) {
     __shared__ float red[17];
     const long r = blockIdx.x;
     const int g = blockIdx.y;
     const XT* xr = x + r * ldx + (long)g * W;
     const ZT* zr = z ? z + r * ldz + (long)g * W : nullptr;
     const bool before = zr && !gate_after;
+    // divisor: one number a (row, group) by which the group's values are divided first
+    const float pre = divisor ? 1.0f / divisor[r * gridDim.y + g] : 1.0f;
     float ss = 0.f;
     for (int c = threadIdx.x; c < W; c += blockDim.x) {
-        float v = to_f32(xr[c]);
+        float v = to_f32(xr[c]) * pre;
         if (before) v *= silu_f(to_f32(zr[c]));
         ss += v * v;
     }
@@ -45,7 +48,7 @@ __global__ __launch_bounds__(256) void rms_norm_groups_kernel(const XT* __restri
     const float rs = 1.0f / sqrtf(ss / (float)W + eps);
     OT* orow = out + r * ldo + (long)g * W;
     for (int c = threadIdx.x; c < W; c += blockDim.x) {
-        float v = to_f32(xr[c]);
+        float v = to_f32(xr[c]) * pre;
         if (before) v *= silu_f(to_f32(zr[c]));
         v *= rs;
         if (weight) v *= weight[(long)g * W + c];
@@ -56,7 +59,8 @@ __global__ __launch_bounds__(256) void rms_norm_groups_kernel(const XT* __restri
 
 extern "C" const char* cpmcu_rms_norm_groups(const void* x, long ldx, int x_dtype, const void* z, long ldz, int z_dtype,
                                              const float* weight, void* out, long ldo, int out_dtype, int n, int groups,
-                                             int W, float eps, int gate_after, hipStream_t stream) {
+                                             int W, float eps, int gate_after, const float* divisor,
+                                             hipStream_t stream) {
     CPMCU_REQUIRE(n > 0 && groups > 0 && W > 0, "rms_norm_groups: empty shape rows=%d groups=%d width=%d", n, groups, W);
     CPMCU_REQUIRE(groups <= 65535, "rms_norm_groups: %d groups exceed the launch grid", groups);
     CPMCU_REQUIRE(ldx >= (long)groups * W && ldo >= (long)groups * W && (!z || ldz >= (long)groups * W),
@@ -65,7 +69,7 @@ extern "C" const char* cpmcu_rms_norm_groups(const void* x, long ldx, int x_dtyp
     const int block = W >= 256 ? 256 : 64;
 #define LAUNCH(XT, ZT, OT)                                                                                     \
     rms_norm_groups_kernel<XT, ZT, OT><<<grid, block, 0, stream>>>((const XT*)x, ldx, (const ZT*)z, ldz, weight, \
-                                                                   (OT*)out, ldo, W, eps, gate_after)
+                                                                   (OT*)out, ldo, W, eps, gate_after, divisor)
     const int zd = z ? z_dtype : x_dtype;
     if (x_dtype == CPMCU_F32 && zd == CPMCU_F32 && out_dtype == CPMCU_F32) LAUNCH(float, float, float);
     else if (x_dtype == CPMCU_F32 && zd == CPMCU_F32 && out_dtype == CPMCU_BF16) LAUNCH(float, float, bf16_t);

@@ -457,11 +457,13 @@ def _ld(t: torch.Tensor, name: str) -> int:
 
 
 def rms_norm_groups(x: torch.Tensor, weight: Optional[torch.Tensor], eps: float, out: torch.Tensor, groups: int = 1,
-                    gate: Optional[torch.Tensor] = None, gate_after: bool = False):
+                    gate: Optional[torch.Tensor] = None, gate_after: bool = False,
+                    divisor: Optional[torch.Tensor] = None):
     """out[r] = v / sqrt(mean(v^2) + eps) * weight, group by group (``groups`` equal parts of a row, each by its
     own root mean square), v = x * silu(gate) when a gate is given (the gate comes before the norm); with
-    ``gate_after`` v = x and the result is multiplied by sigmoid(gate) instead.  x, gate and out may be column
-    slices of wider tensors; statistics in float."""
+    ``gate_after`` v = x and the result is multiplied by sigmoid(gate) instead.  ``divisor`` (float32 [n, groups]):
+    a group's values are divided by its number first.  x, gate and out may be column slices of wider tensors;
+    statistics in float."""
     ldx, ldo = _ld(x, "norm x"), _ld(out, "norm out")
     n, width = x.shape
     if groups <= 0 or width % groups:
@@ -475,11 +477,13 @@ def rms_norm_groups(x: torch.Tensor, weight: Optional[torch.Tensor], eps: float,
         ldz = _ld(gate, "norm gate")
         if tuple(gate.shape) != (n, width):
             raise KernelError(f"norm gate: shape {tuple(gate.shape)}, expected {(n, width)}")
+    if divisor is not None:
+        _need(divisor, "norm divisor", torch.float32, (n, groups))
     _check(_fn("norms", "cpmcu_rms_norm_groups")(_p(x), c_long(ldx), c_int(_code(x)), _p(gate), c_long(ldz),
                                                  c_int(_code(gate) if gate is not None else 0), _p(weight), _p(out),
                                                  c_long(ldo), c_int(_code(out)), c_int(n), c_int(groups),
                                                  c_int(width // groups), c_float(eps), c_int(1 if gate_after else 0),
-                                                 _stream()))
+                                                 _p(divisor), _stream()))
 
 
 def branch_norm_add_norm(x: torch.Tensor, branch: torch.Tensor, branch_weight: torch.Tensor, branch_eps: float,
@@ -736,14 +740,15 @@ def bias_sum(a: torch.Tensor, bias: torch.Tensor, out: torch.Tensor):
 
 def mlstm_scan(proj: torch.Tensor, q_off: int, k_off: int, v_off: int, i_off: int, f_off: int, i_bias: torch.Tensor,
                f_bias: torch.Tensor, cap: float, q_scale: float, S: torch.Tensor, n_state: torch.Tensor,
-               m_state: torch.Tensor, y: torch.Tensor, cu_q: torch.Tensor, seq_slot: torch.Tensor, heads: int, d: int,
-               dv: int, write_state: bool = True):
+               m_state: torch.Tensor, y: torch.Tensor, den: torch.Tensor, cu_q: torch.Tensor, seq_slot: torch.Tensor,
+               heads: int, d: int, dv: int, write_state: bool = True):
     """The matrix-memory recurrence over each sequence's tokens, in float.  proj [n, W] holds, from the given
     columns on, q and k (heads * d each), v (heads * dv) and the raw input and forget gates (heads each); per head
     a = cap tanh((i + i_bias)/cap), b = logsigmoid(cap tanh((f + f_bias)/cap)), m' = max(b + m, a),
-    S' = exp(b + m - m') S + exp(a - m') k v^T, n' likewise with k, y = S'^T q / (max(|n'.q|, exp(-m')) + 1e-6),
-    q multiplied by q_scale.  S float32 [slots, heads, dv, d], n_state [slots, heads, d], m_state [slots, heads];
-    y float32 [n, heads * dv]."""
+    S' = exp(b + m - m') S + exp(a - m') k v^T, n' likewise with k, q multiplied by q_scale.  It leaves the output
+    in two pieces: y = S'^T q (float32 [n, heads * dv]) and den = max(|n'.q|, exp(-m')) + 1e-6 (float32 [n, heads]);
+    the design's output is y / den head by head (rms_norm_groups takes den as its divisor).
+    S float32 [slots, heads, dv, d], n_state [slots, heads, d], m_state [slots, heads]."""
     ld = _ld(proj, "mlstm projection")
     n = proj.shape[0]
     for off, w in ((q_off, heads * d), (k_off, heads * d), (v_off, heads * dv), (i_off, heads), (f_off, heads)):
@@ -755,13 +760,14 @@ def mlstm_scan(proj: torch.Tensor, q_off: int, k_off: int, v_off: int, i_off: in
     _need(n_state, "mlstm normaliser", torch.float32, (S.shape[0], heads, d))
     _need(m_state, "mlstm maximum", torch.float32, (S.shape[0], heads))
     _need(y, "mlstm out", torch.float32, (n, heads * dv))
+    _need(den, "mlstm denominators", torch.float32, (n, heads))
     _need(cu_q, "mlstm sequence starts", torch.int32, (None,))
     B = cu_q.shape[0] - 1
     _need(seq_slot, "mlstm sequence slots", torch.int32, (B,))
     _check(_fn("mlstm", "cpmcu_mlstm_scan")(_p(proj), c_long(ld), c_int(_code(proj)), c_long(q_off), c_long(k_off),
                                             c_long(v_off), c_long(i_off), c_long(f_off), _p(i_bias), _p(f_bias),
                                             c_float(cap), c_float(q_scale), _p(S), _p(n_state), _p(m_state), _p(y),
-                                            _p(cu_q), _p(seq_slot), c_int(B), c_int(heads), c_int(d), c_int(dv),
+                                            _p(den), _p(cu_q), _p(seq_slot), c_int(B), c_int(heads), c_int(d), c_int(dv),
                                             c_int(1 if write_state else 0), _stream()))
 
 

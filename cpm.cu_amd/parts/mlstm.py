@@ -75,14 +75,15 @@ class MLSTMMixer(Mixer):
         with ctx.timed("mlstm_in"):
             u = self.in_proj.forward(h, ctx, "mlstm.in")
         y = ctx.ws.get("mlstm.y", (n, hv), torch.float32)
+        den = ctx.ws.get("mlstm.den", (n, self.heads), torch.float32)
         with ctx.timed("mlstm_scan"):
             ops.mlstm_scan(u, self.q_off, self.k_off, self.v_off, self.i_off, self.f_off, self.i_bias, self.f_bias,
                            self.cap, self.dk ** -0.5, cache.state["memory"], cache.state["normaliser"],
-                           cache.state["maximum"], y, ctx.cu_q, ctx.seq_slot, self.heads, self.dk, self.dv,
+                           cache.state["maximum"], y, den, ctx.cu_q, ctx.seq_slot, self.heads, self.dk, self.dv,
                            write_state=writes_cache)
         gated = ctx.ws.get("mlstm.gated", (n, hv), self.rt.dtype)
         with ctx.timed("mlstm_norm"):
             ops.rms_norm_groups(y, self.norm_w, self.eps, gated, groups=self.heads,
-                                gate=u[:, self.g_off:self.g_off + hv], gate_after=True)
+                                gate=u[:, self.g_off:self.g_off + hv], gate_after=True, divisor=den)
         with ctx.timed("mlstm_out"):
             return self.out_proj.forward(gated, ctx, "mlstm.out", out_dtype=torch.float32, partials=True)

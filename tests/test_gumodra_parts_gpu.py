@@ -244,8 +244,10 @@ def test_matrix_memory_in_portions(dtype, shape):
         for s in live:
             cu.append(cu[-1] + cuts[s][step])
         y = torch.empty(rows.shape[0], H * dv, device=DEV)
+        den = torch.empty(rows.shape[0], H, device=DEV)
         ops.mlstm_scan(dev(rows), offs["q"], offs["k"], offs["v"], offs["i"], offs["f"], dev(i_bias), dev(f_b), cap, d ** -0.5,
-                       S, n_st, m_st, y, i32(cu), i32(live), H, d, dv)
+                       S, n_st, m_st, y, den, i32(cu), i32(live), H, d, dv)
+        y = (y.view(-1, H, dv) / den[:, :, None]).view(-1, H * dv)
         for i, s in enumerate(live):
             got[s].append(y[cu[i]:cu[i + 1]].cpu())
             done[s] += cuts[s][step]
@@ -269,13 +271,14 @@ def test_matrix_memory_remembers_far_back():
         proj[T - 1, 0] = 4.0 * d ** 0.5                                          # the last query asks for feature 0
         proj[:, 2 * d + dv + 1] = f_val
         S, n_st, m_st = torch.zeros(1, H, dv, d, device=DEV), torch.zeros(1, H, d, device=DEV), torch.zeros(1, H, device=DEV)
-        y = torch.empty(T, dv, device=DEV)
+        y, den = torch.empty(T, dv, device=DEV), torch.empty(T, 1, device=DEV)
         z = torch.zeros(1)
         done = 0
         for cut in (500, 399, 1):
             ops.mlstm_scan(dev(proj[done:done + cut]), 0, d, 2 * d, 2 * d + dv, 2 * d + dv + 1, dev(z), dev(z), cap, d ** -0.5,
-                           S, n_st, m_st, y[done:done + cut], i32([0, cut]), i32([0]), H, d, dv)
+                           S, n_st, m_st, y[done:done + cut], den[done:done + cut], i32([0, cut]), i32([0]), H, d, dv)
             done += cut
+        y = y / den
         want = _mlstm_want(proj, z, z, dict(q=0, k=d, v=2 * d, i=2 * d + dv, f=2 * d + dv + 1), H, d, dv, cap)
         close(y, want, "float32", scale=max(float(want.abs().max()), 1.0))
         v0 = proj[0, 2 * d:2 * d + dv]
@@ -293,6 +296,12 @@ def test_head_norm_with_gate_after_it(dtype):
     out = torch.empty(n, H * dv, dtype=DT[dtype], device=DEV)
     ops.rms_norm_groups(dev(y), dev(w), 1e-5, out, groups=H, gate=dev(wide)[:, 10:], gate_after=True)
     want = plain.rms(y.double().view(n, H, dv), 1e-5).reshape(n, -1) * w.double() * torch.sigmoid(wide[:, 10:].double())
+    close(out, want, dtype)
+    # a divisor a (row, head) first: what the recurrence leaves to its norm
+    den = torch.rand(n, H) * 3 + 0.01
+    ops.rms_norm_groups(dev(y), dev(w), 1e-5, out, groups=H, gate=dev(wide)[:, 10:], gate_after=True, divisor=dev(den))
+    want = (plain.rms(y.double().view(n, H, dv) / den.double()[:, :, None], 1e-5).reshape(n, -1) * w.double()
+            * torch.sigmoid(wide[:, 10:].double()))
     close(out, want, dtype)
 
 
