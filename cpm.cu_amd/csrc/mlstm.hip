@@ -14,8 +14,9 @@
 #include "common.h"
 
 // A workgroup of 256 threads walks ML_PB = 256 / ML_L columns; a column's d state values lie over ML_L neighbouring
-// lanes (8 or 16: key index c = l + ML_L i), which sum their shares inside the vector unit.  Keys beyond 128
-// features take 16 lanes a column: twice the workgroups, and half the chain of dependent additions a token.
+// lanes (8 or 32: key index c = l + ML_L i), which sum their shares inside the vector unit.  Keys beyond 128
+// features take 32 lanes a column: four times the workgroups (several a CU, whose walks hide each other's waits)
+// and a quarter of the chain of dependent steps a token.
 
 __device__ inline float log_sigmoid_f(float v) { return fminf(v, 0.f) - log1pf(expf(-fabsf(v))); }
 
@@ -42,7 +43,7 @@ __global__ __launch_bounds__(256) void mlstm_scan_kernel(const T* __restrict__ p
     constexpr int ML_PB = 256 / ML_L;               // columns a workgroup
     constexpr int NS = NR * ML_L;                   // key features, padded
     constexpr int QK = ML_TT * NS / 256;            // q (and k) values a thread brings a tile
-    constexpr int XV = ML_TT * ML_PB / 256;         // v values a thread brings a tile
+    constexpr int XV = (ML_TT * ML_PB + 255) / 256;   // v values a thread brings a tile
     __shared__ float qs[ML_TT][NS];
     __shared__ float ks[ML_TT][NS];
     __shared__ float vs[ML_TT][ML_PB];
@@ -103,7 +104,7 @@ __global__ __launch_bounds__(256) void mlstm_scan_kernel(const T* __restrict__ p
 #pragma unroll
         for (int e2 = 0; e2 < XV; ++e2) {
             const int e = threadIdx.x + e2 * 256;
-            vs[e / ML_PB][e % ML_PB] = rx[e2];
+            if (e < ML_TT * ML_PB) vs[e / ML_PB][e % ML_PB] = rx[e2];
         }
         if ((int)threadIdx.x < tn) {                 // log gates, parked where their exponentials will stand
             take_s[threadIdx.x] = cap * tanhf((ri + bi) * inv_cap);
@@ -138,27 +139,55 @@ __global__ __launch_bounds__(256) void mlstm_scan_kernel(const T* __restrict__ p
         }
         __syncthreads();
         if (t0 + ML_TT < q) fetch(t0 + ML_TT);
+        // a token's keys and queries are asked of LDS while the token before it is worked on
+        float kc[NR], qc[NR], keep_c, tv_c, em_c;
+        auto ask = [&](int tt, float* kk, float* qq, float& keep, float& tv, float& em) {
+#pragma unroll
+            for (int i = 0; i < NR; ++i) {
+                kk[i] = ks[tt][l + ML_L * i];
+                qq[i] = qs[tt][l + ML_L * i];
+            }
+            keep = keep_s[tt];
+            tv = take_s[tt] * vs[tt][pl];
+            em = em_s[tt];
+        };
+        ask(0, kc, qc, keep_c, tv_c, em_c);
+        float* yp = y + (long)(start + t0) * heads * dv + (long)h * dv + p;
+        float* dp = den + (long)(start + t0) * heads + h;
+#pragma unroll 2
         for (int tt = 0; tt < tn; ++tt) {
-            const float keep = keep_s[tt];
-            const float tv = take_s[tt] * vs[tt][pl];
+            float kn[NR], qn[NR], keep_n, tv_n, em_n;
+            ask(min(tt + 1, tn - 1), kn, qn, keep_n, tv_n, em_n);
             float part[4] = {0.f, 0.f, 0.f, 0.f};       // four chains of additions side by side
 #pragma unroll
             for (int i = 0; i < NR; ++i) {
-                const int c = l + ML_L * i;
-                S[i] = keep * S[i] + tv * ks[tt][c];
-                part[i & 3] += S[i] * qs[tt][c];
+                S[i] = keep_c * S[i] + tv_c * kc[i];
+                part[i & 3] += S[i] * qc[i];
             }
             float num = (part[0] + part[1]) + (part[2] + part[3]);
-            // the column's 8 lanes are neighbours: the sum inside the vector unit
+            // the column's lanes are neighbours: the sum inside the vector unit
             num += CPMCU_DPP(num, 0xB1);
             num += CPMCU_DPP(num, 0x4E);
             num += CPMCU_DPP(num, 0x141);
-            if (ML_L == 16) num += CPMCU_DPP(num, 0x140);
-            if (l == 0 && p_ok) {
-                const long t = start + t0 + tt;
-                if (is_n) den[t * heads + h] = fmaxf(fabsf(num), em_s[tt]) + 1e-6f;
-                else y[t * heads * dv + (long)h * dv + p] = num;
+            if (ML_L >= 16) num += CPMCU_DPP(num, 0x140);
+            if (ML_L == 32) {                            // the two rows of 16 lanes that share a column
+                cpmcu_u32x2_t sw = __builtin_amdgcn_permlane16_swap(__float_as_uint(num), __float_as_uint(num), false, false);
+                num = __uint_as_float(sw[0]) + __uint_as_float(sw[1]);
             }
+            if (l == 0 && p_ok) {
+                if (is_n) *dp = fmaxf(fabsf(num), em_c) + 1e-6f;
+                else *yp = num;
+            }
+            yp += (long)heads * dv;
+            dp += heads;
+#pragma unroll
+            for (int i = 0; i < NR; ++i) {
+                kc[i] = kn[i];
+                qc[i] = qn[i];
+            }
+            keep_c = keep_n;
+            tv_c = tv_n;
+            em_c = em_n;
         }
     }
     __syncthreads();
@@ -183,7 +212,7 @@ extern "C" const char* cpmcu_mlstm_scan(const void* proj, long ld, int dtype, lo
     CPMCU_REQUIRE(q_off >= 0 && k_off >= 0 && v_off >= 0 && i_off >= 0 && f_off >= 0 && q_off + (long)heads * d <= ld &&
                   k_off + (long)heads * d <= ld && v_off + (long)heads * dv <= ld && i_off + heads <= ld && f_off + heads <= ld,
                   "mlstm_scan: columns beyond rows of %ld", ld);
-    const int lanes = d > 128 ? 16 : 8, cols = 256 / lanes;
+    const int lanes = d > 128 ? 32 : 8, cols = 256 / lanes;
     const int pb = (dv + 1 + cols - 1) / cols;       // the normaliser is walked as column dv
     CPMCU_REQUIRE(heads <= 65535 && pb <= 65535, "mlstm_scan: shape exceeds the launch grid");
     dim3 grid(n_seqs, heads, pb);
@@ -195,7 +224,7 @@ extern "C" const char* cpmcu_mlstm_scan(const void* proj, long ld, int dtype, lo
                                                                   d, dv, write_state)
 #define BY_NR(Tv)                                  \
     do {                                           \
-        if (lanes == 16) LAUNCH(16, 16, 16, Tv);   \
+        if (lanes == 32) LAUNCH(8, 32, 16, Tv);    \
         else if (need <= 2) LAUNCH(2, 8, 32, Tv);  \
         else if (need <= 4) LAUNCH(4, 8, 32, Tv);  \
         else if (need <= 8) LAUNCH(8, 8, 32, Tv);  \
