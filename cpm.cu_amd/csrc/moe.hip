@@ -1,6 +1,7 @@
 // A feed-forward of routed experts, for steps of any number of tokens and both element types:
 //
-//  * moe_route_kernel: router logits z = Wr h in float (Wr float [E, H]), s = softmax(z); choice scores c = s +
+//  * moe_logits_kernel, moe_select_kernel: router logits z = Wr h in float (Wr float [E, H]), a wavefront a row,
+//    into scratch; then, a wavefront a token: s = softmax(z); choice scores c = s +
 //    correction; the experts form `n_groups` equal groups of neighbours, a group's score is its largest c, and only
 //    experts of the `keep_groups` best groups may be chosen (n_groups = 1: any); the `top` largest c are chosen
 //    (ties: the lower index), their weights are s / (sum of the chosen s + 1e-20).  With w_sg (float [H]) it also
@@ -58,34 +59,40 @@ __device__ inline float lane_dot(const TA* __restrict__ a, const TB* __restrict_
 
 __device__ inline float wave_min_f(float v) { return -wave_max(-v); }
 
-// grid (tokens), 256 or 1024 threads: the wavefronts share the experts' logits, the first one chooses
+// grid (tokens, ceil((E + 1) / 4)), 256 threads: a wavefront a row of the router (row E: the shared expert's gate);
+// logits float [n, E + 1]
 template <typename T>
-__global__ __launch_bounds__(1024) void moe_route_kernel(const T* __restrict__ h, long ldh, const float* __restrict__ wr,
-                                                        const float* __restrict__ correction,
-                                                        const float* __restrict__ w_sg, int H, int E, int n_groups,
-                                                        int keep_groups, int top, int* __restrict__ idx_out,
+__global__ __launch_bounds__(256) void moe_logits_kernel(const T* __restrict__ h, long ldh, const float* __restrict__ wr,
+                                                         const float* __restrict__ w_sg, int H, int E,
+                                                         float* __restrict__ logits) {
+    const long t = blockIdx.x;
+    const int lane = threadIdx.x & 63;
+    const int e = blockIdx.y * 4 + (threadIdx.x >> 6);
+    if (e > E || (e == E && !w_sg)) return;
+    const T* hr = h + t * ldh;
+    const float* row = e < E ? wr + (long)e * H : w_sg;
+    const bool vec = (H % 8 == 0) && (ldh % 8 == 0) && ((uintptr_t)h % 32 == 0) && ((uintptr_t)row % 32 == 0);
+    const float s = wave_sum(lane_dot<T, float>(hr, row, H, lane, vec));
+    if (lane == 0) logits[t * (E + 1) + e] = s;
+}
+
+// grid (tokens), 64 threads: softmax, groups, the top choices and their weights from a row of logits
+__global__ __launch_bounds__(64) void moe_select_kernel(const float* __restrict__ logits,
+                                                        const float* __restrict__ correction, int has_sg, int E,
+                                                        int n_groups, int keep_groups, int top, int* __restrict__ idx_out,
                                                         float* __restrict__ w_out, float* __restrict__ sg_out) {
     __shared__ float z[MOE_MAX_EXPERTS];      // logits, then softmax scores
     __shared__ float c[MOE_MAX_EXPERTS];      // choice scores; -inf once an expert is chosen or shut out
     __shared__ float gs[MOE_MAX_EXPERTS];     // group scores
     const long t = blockIdx.x;
-    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
-    const T* hr = h + t * ldh;
-    const bool vec = (H % 8 == 0) && (ldh % 8 == 0) && ((uintptr_t)h % 32 == 0) && ((uintptr_t)wr % 32 == 0);
-    const int n_waves = blockDim.x >> 6;
-    for (int e = wave; e < E + (w_sg ? 1 : 0); e += n_waves) {
-        const float* row = e < E ? wr + (long)e * H : w_sg;
-        const bool v = vec && (e < E || (uintptr_t)w_sg % 32 == 0);
-        const float s = wave_sum(lane_dot<T, float>(hr, row, H, lane, v));
-        if (lane == 0) {
-            if (e < E) z[e] = s;
-            else sg_out[t] = 1.0f / (1.0f + expf(-s));
-        }
-    }
-    __syncthreads();
-    if (wave != 0) return;
+    const int lane = threadIdx.x;
+    const float* zr = logits + t * (E + 1);
+    if (has_sg && lane == 0) sg_out[t] = 1.0f / (1.0f + expf(-zr[E]));
     float mx = -INFINITY;
-    for (int e = lane; e < E; e += 64) mx = fmaxf(mx, z[e]);
+    for (int e = lane; e < E; e += 64) {
+        z[e] = zr[e];
+        mx = fmaxf(mx, z[e]);
+    }
     mx = wave_max(mx);
     float sum = 0.f;
     for (int e = lane; e < E; e += 64) {
@@ -148,24 +155,25 @@ __global__ __launch_bounds__(1024) void moe_route_kernel(const T* __restrict__ h
 
 extern "C" const char* cpmcu_moe_route(const void* h, long ldh, int dtype, const float* wr, const float* correction,
                                        const float* w_sg, int n, int H, int E, int n_groups, int keep_groups, int top,
-                                       int* idx_out, float* w_out, float* sg_out, hipStream_t stream) {
-    CPMCU_REQUIRE(n > 0 && H > 0 && E > 0, "moe_route: empty shape");
+                                       float* logits, int* idx_out, float* w_out, float* sg_out, hipStream_t stream) {
+    CPMCU_REQUIRE(n > 0 && H > 0 && E > 0 && logits, "moe_route: empty shape");
     CPMCU_REQUIRE(E <= MOE_MAX_EXPERTS, "moe_route: %d experts (up to %d are taken)", E, MOE_MAX_EXPERTS);
     CPMCU_REQUIRE(n_groups >= 1 && E % n_groups == 0 && keep_groups >= 1 && keep_groups <= n_groups,
                   "moe_route: %d experts in %d groups of which %d may be chosen from", E, n_groups, keep_groups);
     CPMCU_REQUIRE(top >= 1 && top <= keep_groups * (E / n_groups), "moe_route: %d experts a token of %d that may be chosen",
                   top, keep_groups * (E / n_groups));
     CPMCU_REQUIRE(!w_sg || sg_out, "moe_route: a place for the shared gate is missing");
-    const int block = E + 1 > 16 ? 1024 : 256;
+    dim3 grid(n, (E + 1 + 3) / 4);
     if (dtype == CPMCU_F32)
-        moe_route_kernel<float><<<n, block, 0, stream>>>((const float*)h, ldh, wr, correction, w_sg, H, E, n_groups,
-                                                       keep_groups, top, idx_out, w_out, sg_out);
+        moe_logits_kernel<float><<<grid, 256, 0, stream>>>((const float*)h, ldh, wr, w_sg, H, E, logits);
     else if (dtype == CPMCU_BF16)
-        moe_route_kernel<bf16_t><<<n, block, 0, stream>>>((const bf16_t*)h, ldh, wr, correction, w_sg, H, E, n_groups,
-                                                        keep_groups, top, idx_out, w_out, sg_out);
+        moe_logits_kernel<bf16_t><<<grid, 256, 0, stream>>>((const bf16_t*)h, ldh, wr, w_sg, H, E, logits);
     else
         CPMCU_FAIL("moe_route: unknown dtype %d", dtype);
-    CPMCU_LAUNCH_CHECK("moe_route");
+    CPMCU_LAUNCH_CHECK("moe_logits");
+    moe_select_kernel<<<n, 64, 0, stream>>>(logits, correction, w_sg ? 1 : 0, E, n_groups, keep_groups, top, idx_out, w_out,
+                                            sg_out);
+    CPMCU_LAUNCH_CHECK("moe_select");
     return nullptr;
 }
 

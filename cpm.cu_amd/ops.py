@@ -776,12 +776,13 @@ MOE_MAX_EXPERTS = 1024
 
 def moe_route(h: torch.Tensor, router: torch.Tensor, correction: Optional[torch.Tensor], shared_gate: Optional[torch.Tensor],
               n_groups: int, keep_groups: int, top: int, idx: torch.Tensor, weights: torch.Tensor,
-              shared_out: Optional[torch.Tensor] = None):
+              shared_out: Optional[torch.Tensor] = None, logits: Optional[torch.Tensor] = None):
     """Routing of every token to ``top`` of E experts.  Logits router . h in float (router float32 [E, H]), scores
     s = softmax; choice scores s + correction; the experts form n_groups equal groups of neighbours, of which only
     the keep_groups with the largest best choice score may be chosen from; the top largest choice scores win (ties:
     the lower index); weights = s of the chosen / (their sum + 1e-20).  idx int32 [n, top], weights float32 [n, top].
-    shared_gate (float32 [H]): shared_out[t] = sigmoid(shared_gate . h[t])."""
+    shared_gate (float32 [H]): shared_out[t] = sigmoid(shared_gate . h[t]).  logits: float32 [n, E + 1] of scratch
+    (allocated here when absent: a caller that must not allocate brings it)."""
     ldh = _ld(h, "router input")
     n, H = h.shape
     _need(router, "router weight", torch.float32, (None, H))
@@ -793,9 +794,12 @@ def moe_route(h: torch.Tensor, router: torch.Tensor, correction: Optional[torch.
         _need(shared_out, "shared gate", torch.float32, (n,))
     _need(idx, "chosen experts", torch.int32, (n, top))
     _need(weights, "expert weights", torch.float32, (n, top))
+    if logits is None:
+        logits = torch.empty((n, E + 1), dtype=torch.float32, device=h.device)
+    _need(logits, "router logits", torch.float32, (n, E + 1))
     _check(_fn("moe", "cpmcu_moe_route")(_p(h), c_long(ldh), c_int(_code(h)), _p(router), _p(correction), _p(shared_gate),
                                          c_int(n), c_int(H), c_int(E), c_int(n_groups), c_int(keep_groups), c_int(top),
-                                         _p(idx), _p(weights), _p(shared_out), _stream()))
+                                         _p(logits), _p(idx), _p(weights), _p(shared_out), _stream()))
 
 
 def moe_gated(h: torch.Tensor, gate_up: torch.Tensor, idx: torch.Tensor, act: torch.Tensor):

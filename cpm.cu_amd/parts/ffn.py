@@ -145,9 +145,10 @@ class RoutedExpertsFFN(FeedForward):
         idx = ctx.ws.get("moe.idx", (n, self.top), torch.int32)
         wts = ctx.ws.get("moe.weights", (n, self.top), torch.float32)
         sg = ctx.ws.get("moe.shared_gate", (n,), torch.float32) if self.shared is not None else None
+        logits = ctx.ws.get("moe.logits", (n, self.experts + 1), torch.float32)
         with ctx.timed("moe_route"):
             ops.moe_route(h, self.router, self.correction, self.shared_scale, self.groups[0], self.groups[1], self.top,
-                          idx, wts, sg)
+                          idx, wts, sg, logits)
         shared = self.shared.forward(h, ctx) if self.shared is not None else None
         act = ctx.ws.get("moe.act", (n, self.top, self.expert_size), self.rt.dtype)
         out = ctx.ws.get("moe.out", (n, self.hidden_size), torch.float32)
