@@ -207,7 +207,7 @@ extern "C" const char* cpmcu_mlstm_scan(const void* proj, long ld, int dtype, lo
                                         float* den, const int* cu_q, const int* seq_slot, int n_seqs, int heads, int d, int dv,
                                         int write_state, hipStream_t stream) {
     CPMCU_REQUIRE(n_seqs > 0 && heads > 0 && d > 0 && dv > 0, "mlstm_scan: empty shape");
-    CPMCU_REQUIRE(d <= 256, "mlstm_scan: a key size of %d is not supported (at most 256)", d);
+    CPMCU_REQUIRE(d <= 1024, "mlstm_scan: a key size of %d is not supported (at most 1024)", d);
     CPMCU_REQUIRE(cap > 0.f, "mlstm_scan: gate cap %g", cap);
     CPMCU_REQUIRE(q_off >= 0 && k_off >= 0 && v_off >= 0 && i_off >= 0 && f_off >= 0 && q_off + (long)heads * d <= ld &&
                   k_off + (long)heads * d <= ld && v_off + (long)heads * dv <= ld && i_off + heads <= ld && f_off + heads <= ld,
@@ -224,7 +224,9 @@ extern "C" const char* cpmcu_mlstm_scan(const void* proj, long ld, int dtype, lo
                                                                   d, dv, write_state)
 #define BY_NR(Tv)                                  \
     do {                                           \
-        if (lanes == 32) LAUNCH(8, 32, 16, Tv);    \
+        if (lanes == 32 && need <= 8) LAUNCH(8, 32, 16, Tv);        \
+        else if (lanes == 32 && need <= 16) LAUNCH(16, 32, 8, Tv);  \
+        else if (lanes == 32) LAUNCH(32, 32, 4, Tv);                \
         else if (need <= 2) LAUNCH(2, 8, 32, Tv);  \
         else if (need <= 4) LAUNCH(4, 8, 32, Tv);  \
         else if (need <= 8) LAUNCH(8, 8, 32, Tv);  \

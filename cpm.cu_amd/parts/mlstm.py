@@ -35,8 +35,8 @@ class MLSTMMixer(Mixer):
                  gate_cap: float, eps: float):
         """``names``: checkpoint tensors for 'q', 'k', 'v', 'gate', 'input_gate', 'input_gate_bias', 'forget_gate',
         'forget_gate_bias', 'norm', 'out'."""
-        if key_dim > 256:
-            raise ValueError(f"mlstm: a key size of {key_dim} is not supported (at most 256)")
+        if key_dim > 1024:
+            raise ValueError(f"mlstm: a key size of {key_dim} is not supported (at most 1024)")
         if gate_cap <= 0:
             raise ValueError(f"mlstm: gate cap {gate_cap}")
         self.names = dict(names)

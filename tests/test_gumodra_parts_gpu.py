@@ -223,7 +223,8 @@ def _mlstm_want(proj, i_bias, f_b, offs, H, d, dv, cap):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("shape", [(3, 16, 24), (1, 40, 8), (2, 12, 7), (6, 32, 48), (2, 130, 70), (1, 256, 33)])
+@pytest.mark.parametrize("shape", [(3, 16, 24), (1, 40, 8), (2, 12, 7), (6, 32, 48), (2, 130, 70), (1, 256, 33), (2, 300, 9),
+                                   (1, 1000, 5)])
 def test_matrix_memory_in_portions(dtype, shape):
     """Two sequences in slots 2 and 0, fed in portions of unequal sizes (down to one token, across a tile of 32):
     equal to the recurrence over each whole sequence; other slots stay untouched."""
