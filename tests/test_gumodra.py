@@ -202,7 +202,7 @@ def _cache(window, keep_first, max_tokens=64 * 40, slots=3, page=32, step=50):
     return SequenceCache(needs, max_tokens, slots, 4096, page, "cpu", torch.float32, step)
 
 
-@pytest.mark.parametrize("window, keep_first", [(40, 20), (33, 70), (100, 0), (5, 32), (64, 1)])
+@pytest.mark.parametrize("window, keep_first", [(44, 18), (33, 70), (100, 0), (5, 32), (64, 1)])
 def test_window_group_keeps_what_its_queries_read(window, keep_first):
     c = _cache(window, keep_first)
     g = c.groups[0]
@@ -234,7 +234,7 @@ def test_room_for_counts_as_extend_does():
     from cpmcu_amd.cache.paged import CacheError
     rnd = random.Random(11)
     for trial in range(30):
-        window, keep_first = rnd.choice([(40, 20), (33, 70), (20, 0), (70, 33)])
+        window, keep_first = rnd.choice([(44, 18), (33, 70), (20, 0), (70, 33)])
         c = _cache(window, keep_first, max_tokens=32 * rnd.choice([6, 9, 14]), slots=3, step=2048)
         slots = [c.acquire() for _ in range(3)]
         for _ in range(40):

@@ -97,7 +97,7 @@ def test_projection_to_normed_rotated_heads_with_keys_as_values(dtype, shape):
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("shape", [(4, 2, 32, 24, 5, 32), (6, 1, 16, 70, 0, 64), (2, 2, 48, 33, 70, 64), (5, 5, 20, 17, 3, 32),
-                                   (8, 2, 128, 40, 20, 64), (3, 1, 24, 0, 0, 32)])
+                                   (8, 4, 128, 48, 12, 64), (3, 1, 24, 0, 0, 32)])
 def test_window_kept_tokens_and_sink(dtype, shape):
     from cpmcu_amd import ops
     H, G, d, window, keep, page = shape
@@ -126,7 +126,7 @@ def test_matrix_core_prompt_tiles_with_a_window():
     """Prompts of more than 256 tokens whose kv heads serve few query heads put consecutive tokens into one tile:
     the tile's tokens have windows of their own."""
     from cpmcu_amd import ops
-    H, G, d, window, keep, page = 4, 2, 32, 40, 20, 64
+    H, G, d, window, keep, page = 4, 2, 32, 50, 10, 64
     torch.manual_seed(23)
     T = 400
     q, k, v = (torch.randn(T, n, d).to(torch.bfloat16) for n in (H, G, G))
@@ -150,7 +150,7 @@ def test_one_key_that_stands_out_at_the_edges_of_the_window(dtype):
     H, G, d, page = 2, 1, 32, 64
     T = 520
     torch.manual_seed(24)
-    cases = [(40, 20, 100), (40, 20, 19), (40, 20, 20), (64, 0, 64), (64, 0, 63), (33, 70, 69), (33, 70, 70), (100, 3, 2),
+    cases = [(44, 18, 100), (44, 18, 17), (44, 18, 18), (64, 0, 64), (64, 0, 63), (33, 70, 69), (33, 70, 70), (100, 3, 2),
              (100, 3, 300), (1, 0, 77), (500, 0, 10)]
     for window, keep, star in cases:
         k = torch.randn(T, G, d) * 0.1
@@ -223,7 +223,7 @@ def _mlstm_want(proj, i_bias, f_b, offs, H, d, dv, cap):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("shape", [(3, 16, 24), (1, 40, 8), (2, 12, 7), (6, 32, 48), (2, 130, 70), (1, 256, 33), (2, 300, 9),
+@pytest.mark.parametrize("shape", [(3, 16, 24), (1, 40, 8), (2, 12, 7), (5, 32, 40), (2, 130, 70), (1, 256, 33), (2, 300, 9),
                                    (1, 1000, 5)])
 def test_matrix_memory_in_portions(dtype, shape):
     """Two sequences in slots 2 and 0, fed in portions of unequal sizes (down to one token, across a tile of 32):
@@ -309,7 +309,7 @@ def test_head_norm_with_gate_after_it(dtype):
 # ---------------------------------------------------------------------------
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 @pytest.mark.parametrize("shape", [(96, 8, 3, (4, 2)), (100, 6, 2, (3, 3)), (64, 5, 1, None), (128, 64, 6, (8, 3)), (72, 4, 2, (2, 1)),
-                                   (256, 16, 4, (4, 3))])
+                                   (192, 12, 3, (4, 3))])
 def test_routing(dtype, shape):
     from cpmcu_amd import ops
     Hd, E, top, groups = shape
@@ -335,7 +335,7 @@ def test_routing(dtype, shape):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("shape", [(96, 40, 8, 3), (100, 20, 6, 2), (64, 24, 5, 1), (128, 64, 16, 4)])
+@pytest.mark.parametrize("shape", [(96, 40, 8, 3), (100, 20, 6, 2), (64, 24, 5, 1), (128, 56, 12, 4)])
 def test_experts(dtype, shape):
     from cpmcu_amd import ops
     Hd, F, E, top = shape
@@ -365,7 +365,7 @@ def test_experts(dtype, shape):
     close(out2, want - sgate.double()[:, None] * shared.double().sum(0), "float32" if dtype == "float32" else "bfloat16")
 
 
-@pytest.mark.parametrize("shape", [(96, 40, 8, 3, 300), (104, 24, 6, 2, 65), (64, 24, 5, 1, 700), (128, 64, 16, 4, 1000),
+@pytest.mark.parametrize("shape", [(96, 40, 8, 3, 300), (104, 24, 6, 2, 65), (64, 24, 5, 1, 700), (128, 72, 12, 4, 1000),
                                    (256, 136, 40, 6, 129)])
 def test_experts_of_many_tokens_on_the_matrix_cores(shape):
     """Pairs grouped by expert in tiles of 64 rows: equal to the few-token kernels pair by pair, whatever row of a
